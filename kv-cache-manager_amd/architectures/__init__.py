@@ -1,2 +1,3 @@
 """Architectures known to the engine.  Importing this package registers them."""
 from . import llama  # noqa: F401
+from . import kasuvik  # noqa: F401

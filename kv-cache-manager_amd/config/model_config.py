@@ -27,8 +27,10 @@ def read_config_json(model_dir):
     with open(path) as f:
         raw = json.load(f)
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str):      # some model folders name one class, as a string
+        archs = [raw["architecture"]]
     if not archs or not isinstance(archs, list) or not isinstance(archs[0], str):
-        raise ConfigError(f"{path}: 'architectures' must name the model class, e.g. [\"LlamaForCausalLM\"]")
+        raise ConfigError(f"{path}: 'architectures' (or 'architecture') must name the model class, e.g. [\"LlamaForCausalLM\"]")
     return archs[0], raw
 
 

@@ -1,0 +1,300 @@
+// Attention over a sliding window of tokens and, beside them, one pooled key and value for every
+// block of P tokens that lies wholly before the window; rotary positions by interleaved pairs on the
+// first dims of a head; keys and values of different sizes.
+//
+//   row at position i sees   tokens j with 0 <= i - j < window
+//                            blocks b with b*P + P - 1 <= i - window   (mean key, mean value of its P tokens)
+//   and all of them share one softmax; score = (q . k) * scale_h with a factor per query head.
+//
+// Pages: keys [pages, kv_heads, B, d], values transposed [pages, kv_heads, dv, B] (as the other
+// attentions of this library keep them).  Pooled entries are 32-bit and live with the page that holds
+// their block's last token: [pages, kv_heads, E, d] and [pages, kv_heads, E, dv] with E = ceil(B / P)
+// entries a page; block b, whose last token e = b*P + P - 1 lies in the sequence's page number e / B,
+// is entry b - floor((e / B) * B / P) there.  An entry is made by the step that stores its block's last
+// token, from the P keys and values as the pages hold them, added in ascending position: it does not
+// depend on how the prompt was cut.  Giving a page back gives its entries back.
+//
+// One wave per (row, query head); blocks are walked 64 at a time from block 0, tokens 64 at a time in
+// chunks that start at absolute multiples of 64, with a running maximum: a row's result is a fixed
+// sequence of operations on its own keys, whatever else the launch holds and whichever pages it reads.
+#include <cfloat>
+
+#include "common.h"
+#include "kvcm_hip.h"
+
+namespace kvcm {
+
+constexpr int kWpWaves = 4;
+constexpr int kWpMaxValueDim = 512;
+
+// ------------------------------------------------------------------------- angles of a step
+// cos_sin[t, i] = (cos, sin) of position * base^(-2i/dims).  The angle is formed in double precision
+// (a 32-bit product of a position in the thousands loses the low bits of the angle).
+__global__ void rotary_pairs_table_kernel(const int* __restrict__ positions, float2* __restrict__ cos_sin, int T, int half,
+                                          double log_base, int dims) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * half) return;
+  const int t = idx / half, i = idx % half;
+  const double freq = exp(-log_base * (2.0 * i) / double(dims));
+  const double a = double(positions[t]) * freq;
+  cos_sin[idx] = float2{static_cast<float>(cos(a)), static_cast<float>(sin(a))};
+}
+
+// ------------------------------------------------------- rotation and the page write of a step
+// src [T, nh*d + nkv*d + nkv*dv] 32-bit (q | k | v).  q (rotated) -> q_out [T, nh*d]; k (rotated) and v
+// -> their page slot.  The pair (2i, 2i+1), i < rot/2, is turned; the rest passes.
+template <class T>
+__global__ void __launch_bounds__(256)
+    rotate_store_kernel(const float* __restrict__ src, int ld, const float2* __restrict__ cos_sin, int rot,
+                        const int* __restrict__ slots, T* __restrict__ q_out, int ldq, T* __restrict__ kcache,
+                        T* __restrict__ vcache, int nh, int nkv, int d, int dv, int B) {
+  const int row = blockIdx.x;
+  const float* r = src + size_t(row) * ld;
+  const float2* cs = cos_sin + size_t(row) * (rot / 2);
+  const int slot = slots ? slots[row] : -1;
+  for (int e = threadIdx.x; e < (nh + nkv) * d; e += blockDim.x) {
+    const int head = e / d, i = e % d;
+    float x = r[e];
+    if (i < rot) {      // rot is even: the partner i ^ 1 lies inside the rotated part too
+      const float y = r[size_t(head) * d + (i ^ 1)];
+      const float2 a = cs[i / 2];
+      x = (i & 1) ? __fmaf_rn(x, a.x, __fmul_rn(y, a.y)) : __fmaf_rn(x, a.x, -__fmul_rn(y, a.y));
+    }
+    if (head < nh) store_f(q_out + size_t(row) * ldq + e, x);
+    else if (slot >= 0) store_f(kcache + ((size_t(slot / B) * nkv + (head - nh)) * B + slot % B) * d + i, x);
+  }
+  if (slot < 0) return;
+  const float* v = r + size_t(nh + nkv) * d;
+  for (int e = threadIdx.x; e < nkv * dv; e += blockDim.x) {
+    const int head = e / dv, i = e % dv;
+    store_f(vcache + ((size_t(slot / B) * nkv + head) * dv + i) * B + slot % B, v[e]);
+  }
+}
+
+// ------------------------------------------------------------------- pooled entries of a step
+// A row whose position is the last of a block of P makes that block's entry from the pages.
+template <class T>
+__global__ void __launch_bounds__(kWave)
+    pool_update_kernel(const T* __restrict__ kcache, const T* __restrict__ vcache, float* __restrict__ pk,
+                       float* __restrict__ pv, const int* __restrict__ tables, int table_stride,
+                       const int* __restrict__ row_seq, const int* __restrict__ positions, const int* __restrict__ slots,
+                       int nkv, int d, int dv, int B, int P, int E) {
+  const int row = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x;
+  const int slot = slots[row];
+  const int p = positions[row];
+  if (slot < 0 || (p + 1) % P != 0) return;
+  const int* table = tables + size_t(row_seq[row]) * table_stride;
+  const int pgi = p / B;
+  const int entry = p / P - (pgi * B) / P;
+  const size_t at = (size_t(slot / B) * nkv + kvh) * E + entry;
+  const float inv = 1.0f / float(P);
+  for (int i = lane; i < d; i += kWave) {
+    float acc = 0.f;
+    for (int t = p - P + 1; t <= p; ++t)
+      acc += load_f(kcache + ((size_t(table[t / B]) * nkv + kvh) * B + t % B) * d + i);
+    pk[at * d + i] = acc * inv;
+  }
+  for (int i = lane; i < dv; i += kWave) {
+    float acc = 0.f;
+    for (int t = p - P + 1; t <= p; ++t)
+      acc += load_f(vcache + ((size_t(table[t / B]) * nkv + kvh) * dv + i) * B + t % B);
+    pv[at * dv + i] = acc * inv;
+  }
+}
+
+// -------------------------------------------------------------------------------- attention
+template <class T>
+__global__ void __launch_bounds__(kWpWaves* kWave)
+    attention_window_pool_kernel(const T* __restrict__ q, int ldq, T* __restrict__ out, int ldo,
+                                 const T* __restrict__ kcache, const T* __restrict__ vcache,
+                                 const float* __restrict__ pk, const float* __restrict__ pv,
+                                 const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
+                                 const int* __restrict__ ctx_lens, const float* __restrict__ head_scale, long long items,
+                                 int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E) {
+  extern __shared__ float q_lds[];  // [waves][d], q * scale * head_scale[h]
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const long long item = static_cast<long long>(blockIdx.x) * kWpWaves + wave;
+  const bool active = item < items;
+  const int row = active ? static_cast<int>(item / nh) : 0;
+  const int head = active ? static_cast<int>(item % nh) : 0;
+  float* qs = q_lds + wave * d;
+  if (active) {
+    const float f = head_scale ? scale * head_scale[head] : scale;
+    for (int i = lane; i < d; i += kWave) qs[i] = load_f(q + size_t(row) * ldq + size_t(head) * d + i) * f;
+  }
+  __syncthreads();
+  if (!active) return;
+
+  const int kvh = head / (nh / nkv);
+  const int ctx = ctx_lens[row];
+  T* orow = out + size_t(row) * ldo + size_t(head) * dv;
+  if (ctx <= 0) {
+    for (int i = lane; i < dv; i += kWave) store_f(orow + i, 0.f);
+    return;
+  }
+  const int* table = tables + size_t(row_seq[row]) * table_stride;
+  const int first = (window > 0 && ctx > window) ? ctx - window : 0;
+  // blocks that end at or before position (ctx - 1) - window
+  const int blocks = (P > 0 && window > 0 && ctx - window >= P) ? (ctx - window) / P : 0;
+
+  float m = -INFINITY, l = 0.f;
+  float o[kWpMaxValueDim / kWave];
+#pragma unroll
+  for (int i = 0; i < kWpMaxValueDim / kWave; ++i) o[i] = 0.f;
+
+  for (int c0 = 0; c0 < blocks; c0 += kWave) {
+    const int b = c0 + lane;
+    const bool valid = b < blocks;
+    float s = -INFINITY;
+    int page = 0, entry = 0;
+    if (valid) {
+      const int e = b * P + P - 1, pgi = e / B;
+      page = table[pgi];
+      entry = b - (pgi * B) / P;
+      const float* kp = pk + ((size_t(page) * nkv + kvh) * E + entry) * d;
+      s = 0.f;
+      for (int i = 0; i < d; ++i) s = fmaf(qs[i], kp[i], s);
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float alpha = expf(m - m_new);
+    const float p = valid ? expf(s - m_new) : 0.f;
+    l = l * alpha + wave_sum(p);
+#pragma unroll
+    for (int i = 0; i < kWpMaxValueDim / kWave; ++i) o[i] *= alpha;
+    const int n = blocks - c0 < kWave ? blocks - c0 : kWave;
+    for (int j = 0; j < n; ++j) {
+      const float pj = __shfl(p, j, kWave);
+      const int page_j = __shfl(page, j, kWave), entry_j = __shfl(entry, j, kWave);
+      const float* vp = pv + ((size_t(page_j) * nkv + kvh) * E + entry_j) * dv;
+#pragma unroll
+      for (int i = 0; i < kWpMaxValueDim / kWave; ++i) {
+        const int c = lane + i * kWave;
+        if (c < dv) o[i] = fmaf(pj, vp[c], o[i]);
+      }
+    }
+    m = m_new;
+  }
+
+  const size_t khead = size_t(B) * d, kpage = khead * nkv;
+  const size_t vhead = size_t(B) * dv, vpage = vhead * nkv;
+  for (int c0 = (first / kWave) * kWave; c0 < ctx; c0 += kWave) {
+    const int t = c0 + lane;
+    const bool valid = t >= first && t < ctx;
+    float s = -INFINITY;
+    if (valid) {
+      const T* kp = kcache + size_t(table[t / B]) * kpage + kvh * khead + size_t(t % B) * d;
+      s = 0.f;
+      for (int i = 0; i < d; ++i) s = fmaf(qs[i], load_f(kp + i), s);
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float alpha = expf(m - m_new);
+    const float p = valid ? expf(s - m_new) : 0.f;
+    l = l * alpha + wave_sum(p);
+#pragma unroll
+    for (int i = 0; i < kWpMaxValueDim / kWave; ++i) o[i] *= alpha;
+    const int j_lo = first > c0 ? first - c0 : 0;
+    const int j_hi = ctx - c0 < kWave ? ctx - c0 : kWave;
+    for (int j = j_lo; j < j_hi; ++j) {
+      const float pj = __shfl(p, j, kWave);
+      const int tj = c0 + j;
+      const T* vp = vcache + size_t(table[tj / B]) * vpage + kvh * vhead + tj % B;  // [dim][slot]
+#pragma unroll
+      for (int i = 0; i < kWpMaxValueDim / kWave; ++i) {
+        const int c = lane + i * kWave;
+        if (c < dv) o[i] = fmaf(pj, load_f(vp + size_t(c) * B), o[i]);
+      }
+    }
+    m = m_new;
+  }
+#pragma unroll
+  for (int i = 0; i < kWpMaxValueDim / kWave; ++i) {
+    const int c = lane + i * kWave;
+    if (c < dv) store_f(orow + c, o[i] / l);
+  }
+}
+
+}  // namespace kvcm
+
+using namespace kvcm;
+
+extern "C" {
+
+int kvcm_rotary_pairs_table(const int* positions, float* cos_sin, int T, int dims, float base, hipStream_t s) {
+  if (T == 0 || dims == 0) return 0;
+  KVCM_REQUIRE(T > 0 && dims > 0 && dims % 2 == 0 && base > 0.f, "rotary_pairs_table: bad sizes T=%d dims=%d base=%g", T,
+               dims, double(base));
+  const int n = T * (dims / 2);
+  rotary_pairs_table_kernel<<<(n + 255) / 256, 256, 0, s>>>(positions, reinterpret_cast<float2*>(cos_sin), T, dims / 2,
+                                                            log(double(base)), dims);
+  return launch_status("rotary_pairs_table");
+}
+
+int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, const int* slots, void* q_out, int dtype,
+                      int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && d > 0 && dv > 0 && B > 0, "rotate_store: bad sizes");
+  KVCM_REQUIRE(rot % 2 == 0 && rot >= 0 && rot <= d, "rotate_store: %d rotated of %d dims is not supported "
+               "(an even number, at most the head's size)", rot, d);
+  KVCM_REQUIRE(rot == 0 || cos_sin != nullptr, "rotate_store: a rotation needs its table");
+  KVCM_REQUIRE(ld >= (nh + nkv) * d + nkv * dv && ldq >= nh * d, "rotate_store: row strides too small");
+  KVCM_REQUIRE(!slots || (kcache && vcache), "rotate_store: slots without pages");
+  const float2* cs = reinterpret_cast<const float2*>(cos_sin);
+  if (dtype == kF32)
+    rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, cs, rot, slots, static_cast<float*>(q_out), ldq,
+                                                  static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, d, dv, B);
+  else if (dtype == kBF16)
+    rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, cs, rot, slots, static_cast<bf16_t*>(q_out), ldq,
+                                                   static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, d, dv, B);
+  else KVCM_REQUIRE(false, "rotate_store: unknown dtype %d", dtype);
+  return launch_status("rotate_store");
+}
+
+int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* pk, float* pv, const int* tables,
+                     int table_stride, const int* row_seq, const int* positions, const int* slots, int T, int nkv, int d,
+                     int dv, int B, int P, int E, hipStream_t s) {
+  if (T == 0 || P <= 0) return 0;
+  KVCM_REQUIRE(T > 0 && nkv > 0 && d > 0 && dv > 0 && B > 0, "pool_update: bad sizes");
+  KVCM_REQUIRE(E == (B + P - 1) / P, "pool_update: %d entries a page do not fit pages of %d and blocks of %d", E, B, P);
+  KVCM_REQUIRE(nkv <= 65535, "pool_update: too many kv heads");
+  const dim3 grid(T, nkv);
+  if (dtype == kF32)
+    pool_update_kernel<float><<<grid, kWave, 0, s>>>(static_cast<const float*>(kcache), static_cast<const float*>(vcache), pk,
+                                                      pv, tables, table_stride, row_seq, positions, slots, nkv, d, dv, B, P, E);
+  else if (dtype == kBF16)
+    pool_update_kernel<bf16_t><<<grid, kWave, 0, s>>>(static_cast<const bf16_t*>(kcache), static_cast<const bf16_t*>(vcache),
+                                                       pk, pv, tables, table_stride, row_seq, positions, slots, nkv, d, dv, B, P, E);
+  else KVCM_REQUIRE(false, "pool_update: unknown dtype %d", dtype);
+  return launch_status("pool_update");
+}
+
+int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
+                               const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
+                               const int* ctx_lens, const float* head_scale, int T, int nh, int nkv, int d, int dv, int B,
+                               float scale, int window, int P, int E, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && B > 0 && d > 0, "attention_window_pool: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
+  KVCM_REQUIRE(nh % nkv == 0, "attention_window_pool: %d query heads are not a multiple of %d kv heads", nh, nkv);
+  KVCM_REQUIRE(dv > 0 && dv <= kWpMaxValueDim, "attention_window_pool: value size %d is not supported (up to %d)", dv, kWpMaxValueDim);
+  KVCM_REQUIRE(d <= 1024, "attention_window_pool: key size %d is not supported (up to 1024)", d);
+  KVCM_REQUIRE(ldq >= nh * d && ldo >= nh * dv, "attention_window_pool: row strides too small");
+  KVCM_REQUIRE(window >= 0 && P >= 0, "attention_window_pool: negative window or block");
+  KVCM_REQUIRE(P == 0 || (pk && pv && E == (B + P - 1) / P), "attention_window_pool: pooled blocks need their entries");
+  const long long items = static_cast<long long>(T) * nh;
+  const long long blocks = (items + kWpWaves - 1) / kWpWaves;
+  KVCM_REQUIRE(blocks < (1ll << 31), "attention_window_pool: too many rows");
+  const size_t lds = sizeof(float) * kWpWaves * d;
+  if (dtype == kF32)
+    attention_window_pool_kernel<float><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
+        static_cast<const float*>(q), ldq, static_cast<float*>(out), ldo, static_cast<const float*>(kcache),
+        static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, items, nh, nkv, d, dv,
+        B, scale, window, P, E);
+  else if (dtype == kBF16)
+    attention_window_pool_kernel<bf16_t><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
+        static_cast<const bf16_t*>(q), ldq, static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(kcache),
+        static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, items, nh, nkv, d, dv,
+        B, scale, window, P, E);
+  else KVCM_REQUIRE(false, "attention_window_pool: unknown dtype %d", dtype);
+  return launch_status("attention_window_pool");
+}
+
+}  // extern "C"

@@ -1,0 +1,179 @@
+// The generalized delta rule: a matrix state per head that decays per key channel, forgets along the
+// current unit key and learns the current key-value pair,
+//
+//   u = k / sqrt(|k|^2 + 1e-6)
+//   S <- diag(w) S - (a * u) (u^T S) + k v^T        (both terms read the old S)
+//   o = S^T r
+//
+// with w = exp(-exp(-1/2) * sigmoid(w_lin + w0)) and a = sigmoid(a_lin + a_bias) per head and key channel.
+// State, decay, removal rate, unit key and all sums are 32-bit.
+//
+// Two launches.  The first turns the projections of every row into (w, a * u, u), in parallel over rows
+// (the second step of the decay's projection included).
+// The second walks each sequence's run token by token: a workgroup per (sequence, head), a thread per
+// value column j that keeps S[:, j] in registers; per token it needs u^T S[:, j] (a sum over its own
+// registers), updates its column and sums o_j: no thread needs another's column.  The per-token vectors
+// (r, k, w, a*u, u) are staged through LDS a few tokens at a time.  A run that starts at position 0
+// starts from zero without reading its slot.  Tokens are taken one by one in prompts and in decoding.
+#include "common.h"
+#include "kvcm_hip.h"
+
+namespace kvcm {
+
+constexpr int kDeltaTile = 8;      // tokens staged at once
+
+// one wave per (row, head).  The decay's logit is a two-step projection whose second step runs here in 32-bit:
+// w_lin[c] = sum_j w2[c, j] * tanh(low[j]), low = the first step's output (rank values a row).
+constexpr int kDeltaMaxRank = 256;
+__global__ void __launch_bounds__(256)
+    delta_prepare_kernel(const float* __restrict__ k, int ldk, const float* __restrict__ a_lin, int lda,
+                         const float* __restrict__ a_bias, const float* __restrict__ low, int ldlow,
+                         const float* __restrict__ w2, int rank, const float* __restrict__ w0,
+                         float* __restrict__ w_out, float* __restrict__ au_out, float* __restrict__ u_out, long long items,
+                         int heads, int d) {
+  __shared__ float th[256 / kWave][kDeltaMaxRank];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const long long item = static_cast<long long>(blockIdx.x) * (256 / kWave) + wave;
+  const bool active = item < items;
+  const int row = active ? static_cast<int>(item / heads) : 0, head = active ? static_cast<int>(item % heads) : 0;
+  if (active)
+    for (int j = lane; j < rank; j += kWave) th[wave][j] = tanhf(low[size_t(row) * ldlow + j]);
+  __syncthreads();
+  if (!active) return;
+  const size_t col = size_t(head) * d, D = size_t(heads) * d;
+  const float* kr = k + size_t(row) * ldk + col;
+  float ss = 0.f;
+  for (int i = lane; i < d; i += kWave) ss = fmaf(kr[i], kr[i], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss + 1e-6f);
+  const float rate = 0.60653065971263342f;      // exp(-1/2)
+  for (int i = lane; i < d; i += kWave) {
+    const float u = kr[i] * inv;
+    const float a = 1.0f / (1.0f + expf(-(a_lin[size_t(row) * lda + col + i] + a_bias[col + i])));
+    float wl = 0.f;
+    const float* w2r = w2 + (col + i) * rank;
+    for (int j = 0; j < rank; ++j) wl = fmaf(w2r[j], th[wave][j], wl);
+    const float g = 1.0f / (1.0f + expf(-(wl + w0[col + i])));
+    w_out[size_t(row) * D + col + i] = expf(-rate * g);
+    au_out[size_t(row) * D + col + i] = a * u;
+    u_out[size_t(row) * D + col + i] = u;
+  }
+}
+
+template <int DKP>
+__global__ void __launch_bounds__(256)
+    delta_scan_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
+                      const float* __restrict__ v, int ldv, const float* __restrict__ w, const float* __restrict__ au,
+                      const float* __restrict__ u, float* __restrict__ o, int ldo, float* __restrict__ state,
+                      const int* __restrict__ run_start, const int* __restrict__ seq_start,
+                      const int* __restrict__ state_slots, int heads, int dk, int dv) {
+  __shared__ float tile[kDeltaTile][5][DKP];      // r, k, w, a*u, u of the staged tokens (zero beyond dk)
+  const int s = blockIdx.y, head = blockIdx.x;
+  const int j = threadIdx.x;
+  const int r0 = run_start[s], r1 = run_start[s + 1];
+  const int slot = state_slots[s];
+  if (r1 <= r0) return;
+  const size_t D = size_t(heads) * dk;
+  if (slot < 0) {
+    if (j < dv)
+      for (int row = r0; row < r1; ++row) o[size_t(row) * ldo + size_t(head) * dv + j] = 0.f;
+    return;
+  }
+  float* st = state + ((size_t(slot) * heads + head) * dk) * dv + j;      // [slot][head][i][j]
+  const bool fresh = seq_start[s] == 0;
+  float S[DKP];
+#pragma unroll
+  for (int i = 0; i < DKP; ++i) S[i] = (i < dk && j < dv && !fresh) ? st[size_t(i) * dv] : 0.f;
+
+  for (int t0 = r0; t0 < r1; t0 += kDeltaTile) {
+    const int nt = r1 - t0 < kDeltaTile ? r1 - t0 : kDeltaTile;
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * 5 * DKP; e += blockDim.x) {
+      const int t = e / (5 * DKP), which = (e / DKP) % 5, i = e % DKP;
+      const int row = t0 + t;
+      float val = 0.f;
+      if (i < dk) {
+        const size_t col = size_t(head) * dk + i;
+        if (which == 0) val = r[size_t(row) * ldr + col];
+        else if (which == 1) val = k[size_t(row) * ldk + col];
+        else if (which == 2) val = w[size_t(row) * D + col];
+        else if (which == 3) val = au[size_t(row) * D + col];
+        else val = u[size_t(row) * D + col];
+      }
+      tile[t][which][i] = val;
+    }
+    __syncthreads();
+    if (j < dv) {
+      for (int t = 0; t < nt; ++t) {
+        const int row = t0 + t;
+        const float vj = v[size_t(row) * ldv + size_t(head) * dv + j];
+        float sa = 0.f;
+#pragma unroll
+        for (int i = 0; i < DKP; ++i) sa = fmaf(tile[t][4][i], S[i], sa);
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < DKP; ++i) {
+          float sn = tile[t][2][i] * S[i];
+          sn = fmaf(-tile[t][3][i], sa, sn);
+          sn = fmaf(tile[t][1][i], vj, sn);
+          S[i] = sn;
+          acc = fmaf(sn, tile[t][0][i], acc);
+        }
+        o[size_t(row) * ldo + size_t(head) * dv + j] = acc;
+      }
+    }
+  }
+  if (j < dv) {
+#pragma unroll
+    for (int i = 0; i < DKP; ++i)
+      if (i < dk) st[size_t(i) * dv] = S[i];
+  }
+}
+
+}  // namespace kvcm
+
+using namespace kvcm;
+
+extern "C" {
+
+// k, a_lin: 32-bit rows with heads*d columns each (at their own strides); low: 32-bit rows of `rank` columns;
+// w2 [heads*d, rank], a_bias, w0 [heads*d]; w_out, au_out, u_out [T, heads*d]: all 32-bit.
+int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, const float* a_bias, const float* low, int ldlow,
+                       const float* w2, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,
+                       int d, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && heads > 0 && d > 0, "delta_prepare: bad sizes T=%d heads=%d d=%d", T, heads, d);
+  KVCM_REQUIRE(rank > 0 && rank <= kDeltaMaxRank, "delta_prepare: a rank of %d is not supported (1 to %d)", rank, kDeltaMaxRank);
+  KVCM_REQUIRE(ldk >= heads * d && lda >= heads * d && ldlow >= rank, "delta_prepare: row strides too small");
+  const long long items = static_cast<long long>(T) * heads;
+  const long long blocks = (items + 3) / 4;
+  KVCM_REQUIRE(blocks < (1ll << 31), "delta_prepare: too many rows");
+  delta_prepare_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(k, ldk, a_lin, lda, a_bias, low, ldlow, w2, rank, w0, w_out,
+                                                                     au_out, u_out, items, heads, d);
+  return launch_status("delta_prepare");
+}
+
+// r, k [T, heads*dk], v [T, heads*dv] at their own strides; w, au, u [T, heads*dk] dense; o [T, >= heads*dv];
+// state [slots, heads, dk, dv]; all 32-bit.
+int kvcm_delta_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* w, const float* au,
+                    const float* u, float* o, int ldo, float* state, const int* run_start, const int* seq_start,
+                    const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s) {
+  if (S == 0) return 0;
+  KVCM_REQUIRE(S > 0 && heads > 0 && dk > 0 && dv > 0, "delta_scan: bad sizes S=%d heads=%d dk=%d dv=%d", S, heads, dk, dv);
+  KVCM_REQUIRE(dk <= 128 && dv <= 256, "delta_scan: key size %d / value size %d are not supported (up to 128 / 256)", dk, dv);
+  KVCM_REQUIRE(S <= 65535, "delta_scan: too many sequences for one launch (%d)", S);
+  KVCM_REQUIRE(ldr >= heads * dk && ldk >= heads * dk && ldv >= heads * dv && ldo >= heads * dv, "delta_scan: row strides too small");
+  const dim3 grid(heads, S);
+  const int threads = ((dv + kWave - 1) / kWave) * kWave;
+#define KVCM_DELTA(DKP)                                                                                              \
+  delta_scan_kernel<DKP><<<grid, threads, 0, s>>>(r, ldr, k, ldk, v, ldv, w, au, u, o, ldo, state, run_start, seq_start, \
+                                                  state_slots, heads, dk, dv)
+  if (dk <= 16) KVCM_DELTA(16);
+  else if (dk <= 32) KVCM_DELTA(32);
+  else if (dk <= 64) KVCM_DELTA(64);
+  else KVCM_DELTA(128);
+#undef KVCM_DELTA
+  return launch_status("delta_scan");
+}
+
+}  // extern "C"

@@ -425,6 +425,39 @@ __global__ void add_residual_kernel(float* __restrict__ x, const T* __restrict__
     x[i] += load_f(y + i);
 }
 
+
+// ---------------------------------------------------------------- embedding with a factor
+template <class TW>
+__global__ void embed_scaled_kernel(const int* __restrict__ ids, const TW* __restrict__ table, float* __restrict__ x,
+                                    int H, int V, float factor) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* dst = x + size_t(t) * H;
+  if (id < 0 || id >= V) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = 0.f;
+    return;
+  }
+  const TW* src = table + size_t(id) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = load_f(src + i) * factor;
+}
+
+// ------------------------------------------------------------------ gated activation
+// out = act(gate) * up, row = [gate (I) | up (I)] in 32-bit; act: 0 silu, 1 relu, 2 gelu by tanh
+// (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))).  Computed in 32-bit, rounded once.
+template <class TO>
+__global__ void __launch_bounds__(256)
+    gated_act_kernel(const float* __restrict__ gu, int ld, TO* __restrict__ out, int ldo, int I, int act) {
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  const float g = gu[size_t(t) * ld + i], u = gu[size_t(t) * ld + I + i];
+  float a;
+  if (act == 1) a = fmaxf(g, 0.f);
+  else if (act == 2) a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  else a = g / (1.0f + expf(-g));
+  store_f(out + size_t(t) * ldo + i, a * u);
+}
+
 }  // namespace kvcm
 
 using namespace kvcm;
@@ -432,6 +465,28 @@ using namespace kvcm;
 extern "C" {
 
 const char* kvcm_hip_last_error() { return g_hip_error.c_str(); }
+
+int kvcm_embed_scaled(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, float factor,
+                      hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && H > 0 && V > 0, "embed_scaled: bad sizes T=%d H=%d V=%d", T, H, V);
+  if (table_dtype == kF32) embed_scaled_kernel<float><<<T, 256, 0, s>>>(ids, static_cast<const float*>(table), x, H, V, factor);
+  else if (table_dtype == kBF16) embed_scaled_kernel<bf16_t><<<T, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table), x, H, V, factor);
+  else KVCM_REQUIRE(false, "embed_scaled: unknown table dtype %d", table_dtype);
+  return launch_status("embed_scaled");
+}
+
+int kvcm_gated_act(const float* gate_up, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && I > 0 && ld >= 2 * I && ldo >= I, "gated_act: bad sizes T=%d I=%d", T, I);
+  KVCM_REQUIRE(T <= 65535, "gated_act: too many rows for one launch (%d)", T);
+  KVCM_REQUIRE(act >= 0 && act <= 2, "gated_act: unknown activation %d (0 silu, 1 relu, 2 gelu_tanh)", act);
+  const dim3 grid((I + 255) / 256, T);
+  if (out_dtype == kF32) gated_act_kernel<float><<<grid, 256, 0, s>>>(gate_up, ld, static_cast<float*>(out), ldo, I, act);
+  else if (out_dtype == kBF16) gated_act_kernel<bf16_t><<<grid, 256, 0, s>>>(gate_up, ld, static_cast<bf16_t*>(out), ldo, I, act);
+  else KVCM_REQUIRE(false, "gated_act: unknown output dtype %d", out_dtype);
+  return launch_status("gated_act");
+}
 
 int kvcm_embed(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, hipStream_t s) {
   if (T == 0) return 0;

@@ -141,6 +141,49 @@ int kvcm_probe_sums(float* partials, unsigned* counters, float* out, int S, int 
 int kvcm_probe_phases(const void* weights, const long long* phase_bytes, int phases, int layers, int persistent, int G,
                       unsigned* counters, float* act, unsigned* flags, void* sink, int spin_cap, hipStream_t s);
 
+// ---- parts of sequence models beyond the dense decoder ----------------------------------------------
+// (elementwise.hip) the embedding times a factor; act(gate) * up with act 0 silu, 1 relu, 2 gelu by tanh
+int kvcm_embed_scaled(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, float factor,
+                      hipStream_t s);
+int kvcm_gated_act(const float* gate_up, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s);
+// (norm_chain.hip) 32-bit RMS norms chained along a row: two branches combined, normed, added to the stream, the
+// stream normed again; the norm of every head with a weight and a sigmoid gate
+int kvcm_rmsnorm_chain(float* x, const float* a, const float* b, const float* wa, const float* wb, float combine,
+                       const float* w_post, const int* rows, const float* w_pre, void* out, int out_dtype, int R, int H,
+                       float eps, hipStream_t s);
+int kvcm_head_norm_gate(const float* o, int ldo, const float* g, int ldg, const float* w, void* out, int out_dtype,
+                        int ldout, int T, int heads, int d, float eps, hipStream_t s);
+// (short_conv.hip) a short causal convolution per channel over packed runs, its last inputs kept per sequence
+int kvcm_short_conv(const float* in, int ld_in, const float* bias_in, const float* w, const float* bias_out,
+                    const float* state, void* out, int out_dtype, int ld_out, const int* row_seq, const int* positions,
+                    const int* ctx_lens, const int* run_start, const int* seq_start, const int* state_slots, int T, int C,
+                    int taps, int act, hipStream_t s);
+int kvcm_short_conv_state(const float* in, int ld_in, const float* bias_in, float* state, const int* run_start,
+                          const int* seq_start, const int* seq_end, const int* state_slots, int S, int C, int taps,
+                          hipStream_t s);
+// (attention_window_pool.hip) rotation by interleaved pairs, attention over a window and pooled blocks before it
+int kvcm_rotary_pairs_table(const int* positions, float* cos_sin, int T, int dims, float base, hipStream_t s);
+int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, const int* slots, void* q_out, int dtype,
+                      int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B, hipStream_t s);
+int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* pk, float* pv, const int* tables,
+                     int table_stride, const int* row_seq, const int* positions, const int* slots, int T, int nkv, int d,
+                     int dv, int B, int P, int E, hipStream_t s);
+int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
+                               const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
+                               const int* ctx_lens, const float* head_scale, int T, int nh, int nkv, int d, int dv, int B,
+                               float scale, int window, int P, int E, hipStream_t s);
+// (selective_scan.hip, delta_rule.hip) recurrences with a 32-bit state per sequence
+int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
+                        const float* bc, int ldbc, int off_b, int off_c, const float* a_log, const float* dskip,
+                        const float* z, int ldz, void* out, int ldo, float* state, const int* run_start,
+                        const int* seq_start, const int* state_slots, int S, int C, int N, hipStream_t s);
+int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, const float* a_bias, const float* low, int ldlow,
+                       const float* w2, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,
+                       int d, hipStream_t s);
+int kvcm_delta_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* w, const float* au,
+                    const float* u, float* o, int ldo, float* state, const int* run_start, const int* seq_start,
+                    const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s);
+
 // ---- recorded steps ---------------------------------------------------------------------------
 // A step program is the list of launches of one step, recorded once for a step shape and replayed
 // with nothing but the step's metadata changed (the kernels read that from device memory).  The

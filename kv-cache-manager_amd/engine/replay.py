@@ -204,6 +204,8 @@ def main(argv=None):
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--max-live", type=int, default=4,
+                    help="most requests that are live at any time: the pool of state slots is made for that many")
     ap.add_argument("--attn", default="auto", choices=["v1", "v2", "auto"])
     ap.add_argument("--recorded", action="store_true",
                     help="run steps as generation does by default: from launch lists recorded once per step shape")
@@ -212,7 +214,8 @@ def main(argv=None):
     args = ap.parse_args(argv)
     os.makedirs(args.out, exist_ok=True)
     print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
-    rp = TraceReplayer(args.model, args.dtype, args.max_tokens, args.block_size, attn=args.attn, use_programs=args.recorded)
+    rp = TraceReplayer(args.model, args.dtype, args.max_tokens, args.block_size, max_live=args.max_live, attn=args.attn,
+                       use_programs=args.recorded)
     print("[trace_run] ready", file=sys.stderr, flush=True)
     for number, line in enumerate(sys.stdin, 1):
         line = line.strip()

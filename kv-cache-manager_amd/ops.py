@@ -85,6 +85,19 @@ def _declare(lib):
     fn("kvcm_gemm8_supported", i, i, i)
     fn("kvcm_gemm8", vp, i, vp, i, i, i, i, vp, i, f, vp, i, i, i, vp)
     fn("kvcm_gemm8_residual_norm", vp, i, vp, i, i, i, i, vp, vp, i, vp, vp, vp)
+    fn("kvcm_embed_scaled", vp, vp, i, vp, i, i, i, f, vp)
+    fn("kvcm_gated_act", vp, i, vp, i, i, i, i, i, vp)
+    fn("kvcm_rmsnorm_chain", vp, vp, vp, vp, vp, f, vp, vp, vp, vp, i, i, i, f, vp)
+    fn("kvcm_head_norm_gate", vp, i, vp, i, vp, vp, i, i, i, i, i, f, vp)
+    fn("kvcm_short_conv", vp, i, vp, vp, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_short_conv_state", vp, i, vp, vp, vp, vp, vp, vp, i, i, i, vp)
+    fn("kvcm_rotary_pairs_table", vp, vp, i, i, f, vp)
+    fn("kvcm_rotate_store", vp, i, vp, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_pool_update", vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp)
+    fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp)
+    fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
+    fn("kvcm_delta_prepare", vp, i, vp, i, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
+    fn("kvcm_delta_scan", vp, i, vp, i, vp, i, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, vp)
     lib.kvcm_gemm_library_workspace_bytes.restype = C.c_longlong
     lib.kvcm_gemm_library_workspace_bytes.argtypes = []
     lib.kvcm_program_new.restype = vp
@@ -889,3 +902,266 @@ def sample(logits, out, temperature=None, seeds=None, request_ids=None, token_in
         _i32(token_index, "token_index", R)
     _call("kvcm_sample", _ptr(logits), logits.stride(0), _ptr(temperature), _ptr(seeds), _ptr(request_ids),
                              _ptr(token_index), _ptr(out), R, V, _stream())
+
+
+# ------------------------------------------------------------- parts of other sequence models
+GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+
+def _f32(t, name, n=None):
+    if t is None:
+        return
+    _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda, f"{name} must be a contiguous float32 tensor on the GPU")
+    if n is not None:
+        _need(t.numel() >= n, f"{name} holds {t.numel()} values, {n} are needed")
+
+
+def _f32rows(t, name, cols):
+    _need(t.dtype == torch.float32 and t.is_cuda and t.dim() == 2 and t.stride(1) == 1 and t.shape[1] >= cols,
+          f"{name} must be float32 rows of at least {cols} columns")
+
+
+def embed_scaled(ids, table, out, factor):
+    """out[t, :] = float(table[ids[t], :]) * factor."""
+    _dev(ids, table, out)
+    T, H = out.shape
+    _i32(ids, "ids", T)
+    _need(table.dim() == 2 and table.shape[1] == H and table.is_contiguous(), "embedding table must be [V, H]")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "residual stream must be contiguous float32")
+    _call("kvcm_embed_scaled", _ptr(ids), _ptr(table), _DT[table.dtype], _ptr(out), T, H, table.shape[0], float(factor), _stream())
+
+
+def gated_act(gate_up, out, activation):
+    """out[T, I] = act(gate) * up for 32-bit rows [gate (I) | up (I)]; act: "silu", "relu" or "gelu_tanh"."""
+    T, I = out.shape
+    _f32rows(gate_up, "gate_up", 2 * I)
+    _rows2d(out, "out")
+    _need(gate_up.shape[0] >= T and out.is_cuda, "gated_act: the rows do not agree")
+    _need(activation in GATE_ACTIVATIONS, f"unknown activation {activation!r} ({sorted(GATE_ACTIVATIONS)})")
+    _call("kvcm_gated_act", _ptr(gate_up), gate_up.stride(0), _ptr(out), _DT[out.dtype], out.stride(0), T, I,
+          GATE_ACTIVATIONS[activation], _stream())
+
+
+class NormedBranches:
+    """A sublayer's output that is still to be normed and added to the residual stream:
+    x += n(m) * w_post with m = a, or m = combine * (n(a) * wa + n(b) * wb) for two branches side by side
+    (n: division by the root mean square).  ``rmsnorm_chain`` consumes it; ``materialize`` is not offered:
+    the addition belongs to the stream's next reader."""
+
+    def __init__(self, a, w_post, b=None, wa=None, wb=None, combine=1.0):
+        self.a, self.b, self.wa, self.wb, self.combine, self.w_post = a, b, wa, wb, float(combine), w_post
+
+
+def rmsnorm_chain(x, eps, pending=None, weight=None, out=None, rows=None):
+    """x += the pending output (NormedBranches), normed; then out[r] = n(x[src]) * weight, src = rows[r] or r.
+    All arithmetic is 32-bit; ``out`` is rounded once to its dtype.  With ``rows`` the stream is not written."""
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.is_cuda and x.dim() == 2, "x must be contiguous float32 [T, H]")
+    T, H = x.shape
+    a = b = wa = wb = wp = None
+    combine = 1.0
+    if pending is not None:
+        a, b, wa, wb, wp, combine = pending.a, pending.b, pending.wa, pending.wb, pending.w_post, pending.combine
+        for t, n in ((a, "a"), (b, "b")):
+            if t is not None:
+                _need(t.dtype == torch.float32 and t.is_contiguous() and t.shape == x.shape, f"branch {n} must match x")
+        for t in (wa, wb, wp):
+            _f32(t, "a norm weight", H)
+    R = T
+    if out is not None:
+        _need(out.is_cuda and out.is_contiguous() and out.dim() == 2 and out.shape[1] == H, "out must be contiguous [R, H]")
+        _f32(weight, "the norm weight", H)
+        R = out.shape[0]
+        if rows is not None:
+            _i32(rows, "rows", R)
+        else:
+            _need(R <= T, "x has fewer rows than the output")
+    else:
+        _need(pending is not None and rows is None, "rmsnorm_chain: nothing to do")
+    _call("kvcm_rmsnorm_chain", _ptr(x), _ptr(a), _ptr(b), _ptr(wa), _ptr(wb), combine, _ptr(wp), _ptr(rows), _ptr(weight),
+          _ptr(out), _DT[out.dtype] if out is not None else 0, R, H, float(eps), _stream())
+    return out
+
+
+def head_norm_gate(o, gate, weight, out, heads, d, eps):
+    """out[r, h, :] = n(o[r, h, :]) * weight[h, :] * sigmoid(gate[r, h, :])."""
+    T = out.shape[0]
+    _f32rows(o, "o", heads * d)
+    _f32rows(gate, "gate", heads * d)
+    _f32(weight, "weight", heads * d)
+    _rows2d(out, "out")
+    _need(o.shape[0] >= T and gate.shape[0] >= T and out.shape[1] >= heads * d and out.is_cuda, "head_norm_gate: shapes do not agree")
+    _call("kvcm_head_norm_gate", _ptr(o), o.stride(0), _ptr(gate), gate.stride(0), _ptr(weight), _ptr(out), _DT[out.dtype],
+          out.stride(0), T, heads, d, float(eps), _stream())
+    return out
+
+
+def short_conv(x, weight, out, step, state, bias_in=None, bias_out=None, activation=None, rows=None):
+    """Causal convolution per channel over the step's packed runs.  x: 32-bit rows [T, >= C]; weight [C, taps];
+    state [slots, taps-1, C] (the sequences' last inputs, read here); out [T, >= C].  ``step`` brings row_seq,
+    positions, ctx_lens, run_start, seq_start, state_slots."""
+    C, taps = weight.shape
+    T = out.shape[0] if rows is None else rows
+    _f32rows(x, "x", C)
+    _f32(weight, "weight")
+    _f32(bias_in, "bias_in", C)
+    _f32(bias_out, "bias_out", C)
+    _rows2d(out, "out")
+    _need(out.shape[1] >= C and out.is_cuda and x.shape[0] >= T, "short_conv: shapes do not agree")
+    if taps > 1:
+        _need(state is not None and state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 3
+              and tuple(state.shape[1:]) == (taps - 1, C), "state must be float32 [slots, taps-1, C]")
+    _need(activation in (None, "silu"), "short_conv: activation is None or 'silu'")
+    for name in ("row_seq", "positions", "ctx_lens"):
+        _i32(getattr(step, name), name, T)
+    _call("kvcm_short_conv", _ptr(x), x.stride(0), _ptr(bias_in), _ptr(weight), _ptr(bias_out), _ptr(state), _ptr(out),
+          _DT[out.dtype], out.stride(0), _ptr(step.row_seq), _ptr(step.positions), _ptr(step.ctx_lens), _ptr(step.run_start),
+          _ptr(step.seq_start), _ptr(step.state_slots), T, C, taps, 1 if activation == "silu" else 0, _stream())
+    return out
+
+
+def short_conv_state(x, state, step, taps, bias_in=None):
+    """Leaves every sequence's last taps-1 inputs (after this step's rows) in its slot of ``state``."""
+    if taps <= 1:
+        return
+    C = state.shape[2]
+    _f32rows(x, "x", C)
+    _f32(bias_in, "bias_in", C)
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.is_cuda and tuple(state.shape[1:]) == (taps - 1, C),
+          "state must be float32 [slots, taps-1, C]")
+    _call("kvcm_short_conv_state", _ptr(x), x.stride(0), _ptr(bias_in), _ptr(state), _ptr(step.run_start), _ptr(step.seq_start),
+          _ptr(step.seq_end), _ptr(step.state_slots), step.seqs, C, taps, _stream())
+
+
+def rotary_pairs_table(positions, out, dims, base, rows=None):
+    """out[t, i] = (cos, sin) of positions[t] * base^(-2i/dims), float32 [rows, dims/2, 2]."""
+    T = out.shape[0] if rows is None else rows
+    _i32(positions, "positions", T)
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.is_cuda and out.numel() >= T * dims,
+          "the table must be float32 [rows, dims/2, 2]")
+    _call("kvcm_rotary_pairs_table", _ptr(positions), _ptr(out), T, dims, float(base), _stream())
+    return out
+
+
+def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kcache=None, vcache=None, rows=None):
+    """qkv: 32-bit rows [q (nh*d) | k (nkv*d) | v (nkv*dv)].  The first ``rot`` entries of every q and k head are
+    turned by interleaved pairs with the table ``cos_sin``; q goes to q_out [T, nh*d], k and v to their page slots
+    (keys [pages, nkv, B, d], values [pages, nkv, dv, B])."""
+    T = q_out.shape[0] if rows is None else rows
+    _f32rows(qkv, "qkv", (nh + nkv) * d + nkv * dv)
+    _rows2d(q_out, "q_out")
+    _need(q_out.shape[1] >= nh * d and q_out.is_cuda and qkv.shape[0] >= T, "rotate_store: shapes do not agree")
+    B = 1
+    if slots is not None:
+        _i32(slots, "slots", T)
+        _need(kcache is not None and kcache.dtype == q_out.dtype and kcache.is_contiguous() and kcache.dim() == 4
+              and kcache.shape[1] == nkv and kcache.shape[3] == d, "key cache must be [pages, nkv, block_size, d]")
+        B = kcache.shape[2]
+        _need(vcache is not None and vcache.dtype == q_out.dtype and vcache.is_contiguous()
+              and tuple(vcache.shape) == (kcache.shape[0], nkv, dv, B), "value cache must be [pages, nkv, dv, block_size]")
+    if rot:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.numel() >= T * rot,
+              "cos_sin must be float32 [rows, rot/2, 2]")
+    _call("kvcm_rotate_store", _ptr(qkv), qkv.stride(0), _ptr(cos_sin), rot, _ptr(slots), _ptr(q_out), _DT[q_out.dtype],
+          q_out.stride(0), _ptr(kcache), _ptr(vcache), T, nh, nkv, d, dv, B, _stream())
+
+
+def _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P):
+    B = kcache.shape[2]
+    _need(kcache.dim() == 4 and kcache.is_contiguous() and kcache.shape[1] == nkv and kcache.shape[3] == d,
+          "key cache must be [pages, nkv, block_size, d]")
+    _need(vcache.is_contiguous() and tuple(vcache.shape) == (kcache.shape[0], nkv, dv, B) and vcache.dtype == kcache.dtype,
+          "value cache must be [pages, nkv, dv, block_size]")
+    E = 0
+    if P > 0:
+        E = (B + P - 1) // P
+        _need(pk is not None and pk.dtype == torch.float32 and pk.is_contiguous() and tuple(pk.shape) == (kcache.shape[0], nkv, E, d),
+              "pooled keys must be float32 [pages, nkv, ceil(block_size / pool), d]")
+        _need(pv is not None and pv.dtype == torch.float32 and pv.is_contiguous() and tuple(pv.shape) == (kcache.shape[0], nkv, E, dv),
+              "pooled values must be float32 [pages, nkv, ceil(block_size / pool), dv]")
+    return B, E
+
+
+def pool_update(kcache, vcache, pk, pv, tables, table_stride, row_seq, positions, slots, nkv, d, dv, P, rows):
+    """Every row whose position ends a block of P tokens leaves that block's mean key and mean value with its page."""
+    if P <= 0:
+        return
+    _dev(kcache, vcache, pk, pv, tables, row_seq, positions, slots)
+    B, E = _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P)
+    for t, n in ((row_seq, "row_seq"), (positions, "positions"), (slots, "slots")):
+        _i32(t, n, rows)
+    _i32(tables, "tables")
+    _call("kvcm_pool_update", _ptr(kcache), _ptr(vcache), _DT[kcache.dtype], _ptr(pk), _ptr(pv), _ptr(tables), table_stride,
+          _ptr(row_seq), _ptr(positions), _ptr(slots), rows, nkv, d, dv, B, P, E, _stream())
+
+
+def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, row_seq, ctx_lens, nh, nkv, d, dv, scale,
+                          window, P, head_scale=None, rows=None):
+    """out[r, h] = softmax over the last ``window`` tokens and the pooled blocks of P tokens before them
+    (window 0: every token, no blocks) of (q . k) * scale * head_scale[h], times the values."""
+    _dev(q, out, kcache, vcache, tables, row_seq, ctx_lens)
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    T = q.shape[0] if rows is None else rows
+    _need(q.dtype == out.dtype == kcache.dtype, "attention operands must share one dtype")
+    _need(q.shape[1] >= nh * d and out.shape[1] >= nh * dv, "attention rows are too short for the head layout")
+    B, E = _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P)
+    _f32(head_scale, "head_scale", nh)
+    _i32(row_seq, "row_seq", T)
+    _i32(ctx_lens, "ctx_lens", T)
+    _i32(tables, "tables")
+    _call("kvcm_attention_window_pool", _ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
+          _ptr(pk), _ptr(pv), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), _ptr(head_scale), T, nh, nkv, d, dv,
+          B, float(scale), int(window), int(P), E, _stream())
+
+
+def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, state, step):
+    """The selective scan of the step's runs (csrc/hip/selective_scan.hip).  x, out [T, C] in the compute dtype;
+    dt_lin [T, C], bc rows with B at off_b and C at off_c, z rows: 32-bit; state [slots, C, N]."""
+    C, N = a_log.shape
+    _rows2d(x, "x")
+    _rows2d(out, "out")
+    _need(x.dtype == out.dtype and x.is_cuda and x.shape[1] >= C and out.shape[1] >= C, "selective_scan: x and out do not agree")
+    _f32rows(dt_lin, "dt_lin", C)
+    _f32rows(bc, "bc", max(off_b, off_c) + N)
+    _f32rows(z, "z", C)
+    _f32(dt_bias, "dt_bias", C)
+    _f32(a_log, "a_log")
+    _f32(dskip, "dskip", C)
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.is_cuda and tuple(state.shape[1:]) == (C, N),
+          "state must be float32 [slots, C, N]")
+    _call("kvcm_selective_scan", _ptr(x), _DT[x.dtype], x.stride(0), _ptr(dt_lin), dt_lin.stride(0), _ptr(dt_bias), _ptr(bc),
+          bc.stride(0), off_b, off_c, _ptr(a_log), _ptr(dskip), _ptr(z), z.stride(0), _ptr(out), out.stride(0), _ptr(state),
+          _ptr(step.run_start), _ptr(step.seq_start), _ptr(step.state_slots), step.seqs, C, N, _stream())
+    return out
+
+
+def delta_prepare(k, a_lin, a_bias, low, w2, w0, w_out, au_out, u_out, heads, d, rows):
+    """(decay, removal rate times unit key, unit key) of every row and head from the projections; ``low`` is the
+    first step of the decay's projection [T, rank], ``w2`` [heads*d, rank] its second step."""
+    D = heads * d
+    for t, n in ((k, "k"), (a_lin, "a_lin")):
+        _f32rows(t, n, D)
+    rank = w2.shape[1]
+    _f32rows(low, "low", rank)
+    _need(w2.dtype == torch.float32 and w2.is_contiguous() and w2.is_cuda and w2.shape[0] == D, "w2 must be contiguous float32 [heads*d, rank]")
+    for t, n in ((a_bias, "a_bias"), (w0, "w0")):
+        _f32(t, n, D)
+    for t, n in ((w_out, "w_out"), (au_out, "au_out"), (u_out, "u_out")):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and t.shape[0] >= rows and t.shape[1] == D,
+              f"{n} must be contiguous float32 [T, heads*d]")
+    _call("kvcm_delta_prepare", _ptr(k), k.stride(0), _ptr(a_lin), a_lin.stride(0), _ptr(a_bias), _ptr(low), low.stride(0),
+          _ptr(w2), rank, _ptr(w0), _ptr(w_out), _ptr(au_out), _ptr(u_out), rows, heads, d, _stream())
+
+
+def delta_scan(r, k, v, w, au, u, o, state, step, heads, dk, dv):
+    """The delta-rule recurrence over the step's runs (csrc/hip/delta_rule.hip); state [slots, heads, dk, dv]."""
+    for t, n, c in ((r, "r", heads * dk), (k, "k", heads * dk), (v, "v", heads * dv), (o, "o", heads * dv)):
+        _f32rows(t, n, c)
+    for t, n in ((w, "w"), (au, "au"), (u, "u")):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and t.shape[1] == heads * dk, f"{n} must be contiguous float32")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.is_cuda and tuple(state.shape[1:]) == (heads, dk, dv),
+          "state must be float32 [slots, heads, dk, dv]")
+    _call("kvcm_delta_scan", _ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(w), _ptr(au), _ptr(u),
+          _ptr(o), o.stride(0), _ptr(state), _ptr(step.run_start), _ptr(step.seq_start), _ptr(step.state_slots), step.seqs,
+          heads, dk, dv, _stream())
+    return o

@@ -72,10 +72,15 @@ class ParamSpec:
 # ------------------------------------------------------------------------------------ cache
 @dataclass(frozen=True)
 class KVCacheNeed:
-    """Paged keys and values: every key (window 0) or the last ``window`` of them."""
+    """Paged keys and values: every key (window 0) or the last ``window`` of them.  ``value_dim``: the size
+    of a value where it differs from a key's (0: the same).  ``pool`` > 0: beside the tokens, every page keeps
+    one 32-bit mean key and mean value for each block of ``pool`` tokens whose last token it holds
+    (ceil(block_size / pool) entries a page), for attentions that see far blocks as one key."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int = 0
+    pool: int = 0
 
 
 @dataclass(frozen=True)
@@ -226,6 +231,21 @@ class Part:
         """storage: the group's device storage; index: this part's place in it; owner False: the
         cache belongs to another part and is only read."""
         self.cache, self.cache_index, self.cache_owner = storage, index, owner
+
+    # A part that keeps several things per request (pages of keys and values beside a small state, two
+    # states of different shapes) names them: ``cache_needs`` gives {name: need}, and each comes back through
+    # ``attach_named_cache``.  The default is the one unnamed need of ``cache_need``.  Parts that a part
+    # drives itself (``sub_parts``) are asked the same way.
+    def cache_needs(self) -> Dict[str, object]:
+        need = self.cache_need()
+        return {} if need is None else {"": need}
+
+    def attach_named_cache(self, name: str, storage, index: int, owner: bool = True):
+        if name == "":
+            return self.attach_cache(storage, index, owner)
+        if not hasattr(self, "caches"):
+            self.caches = {}
+        self.caches[name] = (storage, index, owner)
 
 
 class Norm(Part):

@@ -247,15 +247,17 @@ class LinearHead(Head):
 
     capturable = True
 
+    def _name(self):
+        return self.params.get("name", self.prefix + "weight")      # name: the table's checkpoint name
+
     def param_specs(self):
         if self.params.get("tied"):
             return []
-        return [ParamSpec("table", ((self.prefix + "weight", (self.params["vocab_size"], self.ctx.hidden_size)),),
-                          role="table")]
+        return [ParamSpec("table", ((self._name(), (self.params["vocab_size"], self.ctx.hidden_size)),), role="table")]
 
     def ignorable_tensors(self):
         # a tied checkpoint may still carry a copy of the shared table
-        return (self.prefix + "weight",) if self.params.get("tied") else ()
+        return (self._name(),) if self.params.get("tied") else ()
 
     def forward(self, step, h, out):
         self.ctx.ops.gemm(h, self.w["table"], out, tuning=step.tune_products)

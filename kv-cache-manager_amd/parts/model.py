@@ -150,6 +150,32 @@ class Model:
             return (head, tail)
         raise ValueError(f"layer {layer.name}: cache_from {src!r} names no layer (a layer's name, or layer.part)")
 
+    @staticmethod
+    def _cache_users(parts):
+        """(slot path, part, need name, need) of everything in a layer that keeps something per request: the
+        layer's parts under their names, the parts they drive themselves under ``name.sub`` (a second level
+        ``name.sub.sub``, and so on: ``sub`` is the index among ``sub_parts()`` unless the parent names its
+        sub-parts in ``sub_part_names``), and a part's named needs under ``path#need``."""
+        out = []
+
+        def walk(path, part):
+            ask = getattr(part, "cache_needs", None)
+            needs = ask() if callable(ask) else {}
+            if not callable(ask):
+                one = getattr(part, "cache_need", None)
+                one = one() if callable(one) else None
+                needs = {} if one is None else {"": one}
+            for name, need in needs.items():
+                out.append((path + ("#" + name if name else ""), part, name, need))
+            subs = list(part.sub_parts()) if hasattr(part, "sub_parts") else []
+            names = getattr(part, "sub_part_names", None) or [str(k) for k in range(len(subs))]
+            for name, sub in zip(names, subs):
+                walk(path + "." + name, sub)
+
+        for slot, part in parts.items():
+            walk(slot, part)
+        return out
+
     def _plan_cache_groups(self) -> List[CacheGroupPlan]:
         groups: List[CacheGroupPlan] = []
         self._cache_of: Dict[Tuple[str, str], Tuple[int, int]] = {}    # owner (layer, part) -> (group, index)
@@ -159,10 +185,7 @@ class Model:
                 unknown = sorted(set(layer.cache_from) - set(parts))
                 if unknown:
                     raise ValueError(f"layer {layer.name}: cache_from names parts the layer does not have: {unknown}")
-            for slot, part in parts.items():
-                need = self._cache_need_of(part)
-                if need is None:
-                    continue
+            for slot, part, _, need in self._cache_users(parts):
                 if not isinstance(need, (KVCacheNeed, StateNeed)):
                     raise TypeError(f"layer {layer.name}, part {slot}: cache_need() must give a KVCacheNeed or a StateNeed")
                 source = self._resolve_cache_source(layer, slot)
@@ -187,15 +210,16 @@ class Model:
         """storages[g]: device storage of group g (see cache.storage).  Every part that reported a
         cache need gets its place (or its owner's, read-only)."""
         for layer, parts in zip(self.spec.layers, self.layer_parts):
-            for slot, part in parts.items():
+            for slot, part, name, _ in self._cache_users(parts):
                 key = (layer.name, slot)
                 owner = self._cache_source.get(key, key)
                 if owner not in self._cache_of:
-                    if self._cache_need_of(part) is not None:
-                        raise RuntimeError(f"layer {layer.name}, part {slot} needs a cache that was not planned")
-                    continue
+                    raise RuntimeError(f"layer {layer.name}, part {slot} needs a cache that was not planned")
                 g, idx = self._cache_of[owner]
-                part.attach_cache(storages[g], idx, owner=owner == key)
+                if name == "" or not hasattr(part, "attach_named_cache"):
+                    part.attach_cache(storages[g], idx, owner=owner == key)
+                else:
+                    part.attach_named_cache(name, storages[g], idx, owner=owner == key)
 
     # --------------------------------------------------------------------------------- step
     def run_layers(self, step):

@@ -1,0 +1,125 @@
+"""Mixers that carry a fixed-size 32-bit state per request instead of keys and values: the selective scan
+(with the short convolution in front of it) and the generalized delta rule.  Their states live in the
+cache manager's state slots; a request's portion that starts at position 0 starts from zero.  Every size,
+constant and tensor name is a parameter.
+"""
+import torch
+
+from ..registry import MIXERS
+from .base import Mixer, ParamSpec, StateNeed
+from .chain_norm_parts import f32_params
+from .llama_parts import _linear
+
+_SMALL = ("conv", "conv_bias", "dt_bias", "a_log", "d_skip", "a_bias", "w0", "w2", "norm")
+
+
+class _StatefulMixer(Mixer):
+    capturable = True
+
+    def bind(self, tensors):
+        small = f32_params({k: v for k, v in tensors.items() if k in _SMALL})
+        super().bind({**tensors, **small})
+
+    def state(self, name):
+        storage, index, _ = self.caches[name]
+        return storage.slots(index)
+
+
+@MIXERS.register("selective_scan")
+class SelectiveScanMixer(_StatefulMixer):
+    """in -> [x | z]; x through a causal convolution (bias, silu); [dt | B | C] = W_x x; dt = softplus(W_dt dt + b);
+    S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n with A = -exp(A_log); y = S C + D x; (y * silu(z)) -> out.
+    params: inner, state, dt_rank, conv (taps).  Tensors under the prefix: in, conv, conv.b, x, dt, dt.b, A_log, D, o.
+    Keeps per request: the convolution's last taps-1 inputs and S, both 32-bit."""
+
+    def param_specs(self):
+        H, p, pre = self.ctx.hidden_size, self.params, self.prefix
+        C, N, R, K = p["inner"], p["state"], p["dt_rank"], p["conv"]
+        return [ParamSpec("w_in", ((pre + "in", (2 * C, H)),)),
+                ParamSpec("conv", ((pre + "conv", (C, K)),)),
+                ParamSpec("conv_bias", ((pre + "conv.b", (C,)),), role="vector"),
+                ParamSpec("w_x", ((pre + "x", (R + 2 * N, C)),)),
+                ParamSpec("w_dt", ((pre + "dt", (C, R)),)),
+                ParamSpec("dt_bias", ((pre + "dt.b", (C,)),), role="vector"),
+                ParamSpec("a_log", ((pre + "A_log", (C, N)),)),
+                ParamSpec("d_skip", ((pre + "D", (C,)),), role="vector"),
+                ParamSpec("w_o", ((pre + "o", (H, C)),))]
+
+    def cache_needs(self):
+        p = self.params
+        needs = {"scan": StateNeed((p["inner"], p["state"]), torch.float32)}
+        if p["conv"] > 1:
+            needs["conv"] = StateNeed((p["conv"] - 1, p["inner"]), torch.float32)
+        return needs
+
+    def flops(self, rows, attended=0):
+        p = self.params
+        return super().flops(rows) + rows * p["inner"] * (6.0 * p["state"] + 2.0 * p["conv"])
+
+    def forward(self, step, h):
+        ops, p, w = self.ctx.ops, self.params, self.w
+        C, N, R, K = p["inner"], p["state"], p["dt_rank"], p["conv"]
+        xz = _linear(self.ctx, step, h, w["w_in"], "scan_xz", dtype=torch.float32)
+        conv_state = self.state("conv") if K > 1 else None
+        x = step.ws("scan_x", (step.rows, C))
+        ops.short_conv(xz, w["conv"], x, step, conv_state, bias_out=w["conv_bias"], activation="silu")
+        ops.short_conv_state(xz, conv_state, step, K)
+        # the step size's low-rank input feeds a product (compute dtype); B and C enter the recurrence (32-bit)
+        low = _linear(self.ctx, step, x, w["w_x"][:R], "scan_dt_low")
+        bc = _linear(self.ctx, step, x, w["w_x"][R:], "scan_bc", dtype=torch.float32)
+        dt = _linear(self.ctx, step, low, w["w_dt"], "scan_dt", dtype=torch.float32)
+        y = step.ws("scan_y", (step.rows, C))
+        ops.selective_scan(x, dt, w["dt_bias"], bc, 0, N, w["a_log"], w["d_skip"], xz[:, C:], y, self.state("scan"), step)
+        return _linear(self.ctx, step, y, w["w_o"], "scan_out", dtype=torch.float32)
+
+
+@MIXERS.register("general_delta")
+class GeneralDeltaMixer(_StatefulMixer):
+    """The generalized delta rule.  r, k, v, g, a (with a bias) and the first step of the decay's projection are
+    one fused product; per head and key channel the decay is w = exp(-exp(-1/2) sigmoid(W_w2 tanh(W_w1 h) + w0)) and
+    the removal rate a = sigmoid(W_a h + b); with u = k / sqrt(|k|^2 + 1e-6):
+    S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r; every head's o is divided by its root mean square, times a
+    weight over all heads, times sigmoid(g), then the output projection.
+    params: heads, dim, eps, rank (of the decay's projection; 0: as the checkpoint has it).
+    Tensors under the prefix: r, k, v, g, a, a.b, w1, w2, w0, norm, o.  Keeps S [heads, dim, dim] per request."""
+
+    def param_specs(self):
+        H, p, pre = self.ctx.hidden_size, self.params, self.prefix
+        D, R = p["heads"] * p["dim"], p.get("rank") or -1
+        return [ParamSpec("w_proj", tuple((pre + n, (D, H)) for n in ("r", "k", "v", "g", "a")) + ((pre + "w1", (R, H)),)),
+                ParamSpec("a_bias", ((pre + "a.b", (D,)),), role="vector"),
+                ParamSpec("w2", ((pre + "w2", (D, R)),)),
+                ParamSpec("w0", ((pre + "w0", (D,)),), role="vector"),
+                ParamSpec("norm", ((pre + "norm", (D,)),), role="vector"),
+                ParamSpec("w_o", ((pre + "o", (H, D)),))]
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        D = self.params["heads"] * self.params["dim"]
+        self.rank = self.w["w2"].shape[1]
+        if self.w["w_proj"].shape[0] != 5 * D + self.rank:
+            raise ValueError(f"general_delta {self.prefix!r}: the two steps of the decay's projection do not agree on their rank "
+                             f"({self.w['w_proj'].shape[0] - 5 * D} and {self.rank})")
+
+    def cache_needs(self):
+        p = self.params
+        return {"delta": StateNeed((p["heads"], p["dim"], p["dim"]), torch.float32)}
+
+    def flops(self, rows, attended=0):
+        p = self.params
+        return super().flops(rows) + rows * p["heads"] * 8.0 * p["dim"] * p["dim"]
+
+    def forward(self, step, h):
+        ops, p, w = self.ctx.ops, self.params, self.w
+        heads, d = p["heads"], p["dim"]
+        D, T = heads * d, step.rows
+        proj = _linear(self.ctx, step, h, w["w_proj"], "delta_proj", dtype=torch.float32)
+        r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
+        low = proj[:, 5 * D:]
+        decay, au, u = (step.ws(n, (T, D), torch.float32) for n in ("delta_w", "delta_au", "delta_u"))
+        ops.delta_prepare(k, a, w["a_bias"], low, w["w2"], w["w0"], decay, au, u, heads, d, T)
+        o = step.ws("delta_o", (T, D), torch.float32)
+        ops.delta_scan(r, k, v, decay, au, u, o, self.state("delta"), step, heads, d, d)
+        gated = step.ws("delta_gated", (T, D))
+        ops.head_norm_gate(o, g, w["norm"], gated, heads, d, p["eps"])
+        return _linear(self.ctx, step, gated, w["w_o"], "delta_out", dtype=torch.float32)

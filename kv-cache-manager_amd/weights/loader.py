@@ -84,10 +84,15 @@ def _stored_dtype(role, stored: torch.dtype, compute: torch.dtype) -> torch.dtyp
     return compute
 
 
+def _fits(stored, declared) -> bool:
+    """A declared size of -1 stands for "as the checkpoint has it" (a size that no configuration key carries)."""
+    return len(stored) == len(declared) and all(d == -1 or d == s for s, d in zip(stored, declared))
+
+
 def check_against(model, source) -> None:
     """Raises one WeightsError listing every missing, unexpected and misshapen tensor."""
     expected, ignorable = {}, set()
-    for part in model.all_parts():
+    for part in model.every_part():
         for spec in part.param_specs():
             for name, shape in spec.sources:
                 expected[name] = tuple(shape)
@@ -95,7 +100,7 @@ def check_against(model, source) -> None:
     have = set(source.names())
     missing = sorted(n for n in expected if n not in have)
     unexpected = sorted(n for n in have if n not in expected and n not in ignorable)
-    wrong = sorted((n, expected[n], source.shape(n)) for n in expected if n in have and source.shape(n) != expected[n])
+    wrong = sorted((n, expected[n], source.shape(n)) for n in expected if n in have and not _fits(source.shape(n), expected[n]))
     if not (missing or unexpected or wrong):
         return
     lines = ["the checkpoint does not fit the model:"]
@@ -113,16 +118,19 @@ def load_weights(model, source, compute_dtype: torch.dtype, device) -> int:
     """Checks, then binds every part's tensors on ``device``.  Returns the bytes now on the device."""
     check_against(model, source)
     total = 0
-    for part in model.all_parts():
+    for part in model.every_part():
         bound = {}
         for spec in part.param_specs():
             dtypes = {_stored_dtype(spec.role, source.dtype(n), compute_dtype) for n, _ in spec.sources}
             if len(dtypes) != 1:
                 raise WeightsError(f"{spec.sources[0][0]} and the tensors fused with it are stored in different precisions")
             dt = dtypes.pop()
-            out = torch.empty(spec.shape, dtype=dt, device=device)
+            shapes = [tuple(source.shape(name)) for name, _ in spec.sources]      # the stored ones: a declared -1 is open
+            if len({sh[1:] for sh in shapes}) != 1:
+                raise WeightsError(f"{spec.sources[0][0]} and the tensors fused with it do not have the same row length")
+            out = torch.empty((sum(sh[0] for sh in shapes),) + shapes[0][1:], dtype=dt, device=device)
             row = 0
-            for name, shape in spec.sources:
+            for (name, _), shape in zip(spec.sources, shapes):
                 out[row:row + shape[0]].copy_(source.get(name).to(dt))
                 row += shape[0]
             bound[spec.name] = out

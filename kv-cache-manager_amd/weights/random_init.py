@@ -108,7 +108,7 @@ def expected_tensors(architecture: str, config) -> Dict[str, tuple]:
     spec = arch.build_spec(config)
     model = Model(spec, BuildContext(torch.float32, torch.device("cpu"), spec.hidden_size, 16, None))
     out = {}
-    for part in model.all_parts():
+    for part in model.every_part():
         for ps in part.param_specs():
             for name, shape in ps.sources:
                 out[name] = (tuple(shape), ps.role)
