@@ -3,11 +3,17 @@
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512] [--layers L]
                   [--sizes tinyllama-1.1b|llama-2-7b|llama-3-8b] [--context-limit 2048] [--prefill-tokens 2048]
                   [--tune-products off|heuristic|all] [--no-points] [--only-prefill]
+  python bench.py --design kasuvik [--design-sizes 2048,4096] [--layers 4] [--prefill-tokens 2048] [--steps K]
 
 A "step" is one decode step of the whole engine (schedule, batch metadata, upload, model step on
 the GPU, sampling, download, update).  W untimed steps, then exactly K timed steps between two
 device synchronisations.  One JSON line is printed: decoded tokens a second at the default batch,
 the same at batch 1 and 64, a 2,048-token prefill, and the decode step's memory roofline.
+
+--design kasuvik leaves that workload alone and measures something else: prefill and decode throughput of the
+Kasuvik decoder (attention over a window and pooled blocks beside a selective scan, and delta-rule layers) at
+layer sizes that resemble served models, beside the Llama decoder at equal width, heads, feed-forward and
+depth, both with random weights through the same engine.  One JSON line with both designs' figures per size.
 """
 import argparse
 import json
@@ -128,6 +134,78 @@ def measured_peaks():
     return out
 
 
+# ------------------------------------------------------------------ another design beside the Llama decoder
+# Layer sizes per width: (heads, kv heads, head size, feed-forward, window, block, scan state, step-size rank, decay rank)
+DESIGN_SIZES = {2048: (32, 4, 64, 5632, 512, 64, 16, 128, 64), 4096: (32, 8, 128, 14336, 1024, 64, 16, 256, 64)}
+
+
+def kasuvik_pair(width, layers, vocab=32000):
+    """(Kasuvik configuration, Llama configuration) of equal width, heads, feed-forward, depth and vocabulary; every
+    fourth layer of the first is a delta-rule layer (the second of each four), the others are parallel layers."""
+    from kvcm_amd.config.kasuvik_config import KasuvikConfig
+    from kvcm_amd.config.model_config import LlamaConfig
+    nh, nkv, hd, ff, window, pool, state, dt_rank, rank = DESIGN_SIZES[width]
+    left = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "conv": 4, "rot": {"dims": hd, "base": 10000.0},
+            "scale": hd ** -0.5, "mask": {"size": window, "pool": pool}}
+    right = {"inner": 2 * width, "state": state, "dt_rank": dt_rank, "conv": 4}
+    listed = []
+    for i in range(layers):
+        if i % 4 == 1:
+            listed.append({"type": "general_delta", "mixer": {"heads": nh, "dim": hd, "rank": rank}, "mlp": {"kind": "dense", "ff": ff}})
+        else:
+            listed.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": {"kind": "dense", "ff": ff}})
+    kas = KasuvikConfig.from_dict({"architecture": "Kasuvik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+                                   "norm": {"eps": 1e-6}, "layers": listed})
+    llama = LlamaConfig.from_dict(dict(vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
+                                       num_attention_heads=nh, num_key_value_heads=nkv, head_dim=hd, max_position_embeddings=8192,
+                                       rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False))
+    return kas, llama
+
+
+def design_main(args):
+    import torch
+    from kvcm_amd.config.engine_config import EngineConfig
+    from kvcm_amd.engine.engine import Engine
+    from kvcm_amd.weights.random_init import random_tensors
+    layers = args.layers or 4
+    T = args.prefill_tokens
+    steps, warmup = min(args.steps, 64), min(args.warmup, 8)
+    limit = max(2048, -(-(T + 64) // 64) * 64, -(-(args.prompt_len + steps + warmup + 64) // 64) * 64)
+    dt = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    record = {"metric": "prefill and decode tok/s of the Kasuvik decoder beside the Llama decoder at equal sizes", "dtype": key,
+              "data": "synthetic", "layers": layers, "prefill_tokens": T, "prompt_len": args.prompt_len, "steps": steps, "sizes": {}}
+    for width in [int(w) for w in args.design_sizes.split(",")]:
+        if width not in DESIGN_SIZES:
+            print("bench.py: unknown width %d for --design-sizes; known: %s" % (width, sorted(DESIGN_SIZES)))
+            sys.exit(2)
+        entry = {}
+        for name, cfg in zip(("kasuvik", "llama"), kasuvik_pair(width, layers)):
+            arch = "Kasuvik" if name == "kasuvik" else "LlamaForCausalLM"
+            tensors = random_tensors(arch, cfg, seed=0, dtype=dt, device="cuda:0")
+            ec = EngineConfig(block_size=16, max_seq_len=limit, num_blocks=8 * limit // 16, max_num_seqs=8,
+                              max_batched_tokens=max(4096, T + 64), dtype=args.dtype, max_logit_rows=64, beyond_max_position=True)
+            eng = Engine(config=ec, architecture=arch, model_config=cfg, tensors=tensors)
+            del tensors
+            V = eng.model.spec.vocab_size
+            sec = prefill_run(eng, T, V)
+            flops = eng.model.step_flops(T, 1, T * (T + 1) // 2 if name == "llama" else T * min(T, DESIGN_SIZES[width][4]))
+            one = {"prefill_tok_s": round(T / sec, 1), "prefill_ms": round(sec * 1e3, 3),
+                   "prefill_flops_frac": round(flops / sec / PEAK_FLOPS[key], 4)}
+            for b in (1, 8):
+                s, c = decode_run(eng, b, args.prompt_len, steps, warmup, V, seed=20 + b)
+                one["decode_b%d_tok_s" % b] = round(b * steps / s, 1)
+                one["decode_b%d_ms" % b] = round(1e3 * s / steps, 4)
+                one["decode_b%d_hbm_frac" % b] = round(eng.runner.step_bytes([c] * b) / (s / steps) / 1e9 / HBM_GBS, 4)
+            entry[name] = one
+            del eng
+            torch.cuda.empty_cache()
+        entry["prefill_ratio"] = round(entry["kasuvik"]["prefill_tok_s"] / entry["llama"]["prefill_tok_s"], 3)
+        entry["decode_b8_ratio"] = round(entry["kasuvik"]["decode_b8_tok_s"] / entry["llama"]["decode_b8_tok_s"], 3)
+        record["sizes"][str(width)] = entry
+    print(json.dumps(record), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,10 +229,17 @@ def main():
                     help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="tokens of the prefill measurement (2,048 in the record; other lengths for sweeps)")
+    ap.add_argument("--design", default="llama", choices=["llama", "kasuvik"],
+                    help="llama: the workload above (the default); kasuvik: prefill and decode of the Kasuvik decoder beside the "
+                         "Llama decoder at equal sizes (--design-sizes, --layers, --prefill-tokens, --prompt-len, --steps)")
+    ap.add_argument("--design-sizes", default="2048,4096", help="widths of the --design comparison (2048, 4096)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N with N > 1 is not supported")
         sys.exit(2)
+
+    if args.design != "llama":
+        return design_main(args)
 
     # a whole prompt fits a step beside the decoding requests
     budget = max(4096, args.prompt_len + args.batch, args.prefill_tokens + 64)

@@ -14,7 +14,7 @@
 // token, from the P keys and values as the pages hold them, added in ascending position: it does not
 // depend on how the prompt was cut.  Giving a page back gives its entries back.
 //
-// One wave per (row, query head); blocks are walked 64 at a time from block 0, tokens 64 at a time in
+// Four waves per (row, query head); blocks are walked 64 at a time from block 0, tokens 64 at a time in
 // chunks that start at absolute multiples of 64, with a running maximum: a row's result is a fixed
 // sequence of operations on its own keys, whatever else the launch holds and whichever pages it reads.
 #include <cfloat>
@@ -103,113 +103,189 @@ __global__ void __launch_bounds__(kWave)
 }
 
 // -------------------------------------------------------------------------------- attention
+// dot of a 32-bit vector (LDS) with a stored row, 16 bytes of the row at a time where its length allows
+template <class T> struct RowPiece;
+template <> struct RowPiece<float> { static constexpr int N = 4; };
+template <> struct RowPiece<bf16_t> { static constexpr int N = 8; };
+
+__device__ __forceinline__ void unpack_piece(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+__device__ __forceinline__ void unpack_piece(const bf16_t* p, float* f) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  f[0] = bf16_bits_to_float(v.x & 0xffffu); f[1] = bf16_bits_to_float(v.x >> 16);
+  f[2] = bf16_bits_to_float(v.y & 0xffffu); f[3] = bf16_bits_to_float(v.y >> 16);
+  f[4] = bf16_bits_to_float(v.z & 0xffffu); f[5] = bf16_bits_to_float(v.z >> 16);
+  f[6] = bf16_bits_to_float(v.w & 0xffffu); f[7] = bf16_bits_to_float(v.w >> 16);
+}
+
+template <class T>
+__device__ __forceinline__ float dot_row(const float* qs, const T* kp, int d, bool wide) {
+  constexpr int N = RowPiece<T>::N;
+  float s = 0.f;
+  if (wide) {
+    for (int i = 0; i < d; i += N) {
+      float f[N];
+      unpack_piece(kp + i, f);
+#pragma unroll
+      for (int e = 0; e < N; ++e) s = fmaf(qs[i + e], f[e], s);
+    }
+  } else {
+    for (int i = 0; i < d; ++i) s = fmaf(qs[i], load_f(kp + i), s);
+  }
+  return s;
+}
+
+// One workgroup of four waves per (row, query head).  The row's chunks (pooled blocks 64 at a time from block 0,
+// then tokens in chunks that start at absolute multiples of 64) are dealt to the waves in turn by their number;
+// each wave keeps a running maximum over its chunks and the four results are merged at the end in wave order.
+// Inside a chunk a lane takes one key for the scores; for the values a lane takes value columns and reads the
+// tokens of its column 16 bytes at a time (values are stored transposed: a column's tokens lie side by side).
 template <class T>
 __global__ void __launch_bounds__(kWpWaves* kWave)
     attention_window_pool_kernel(const T* __restrict__ q, int ldq, T* __restrict__ out, int ldo,
                                  const T* __restrict__ kcache, const T* __restrict__ vcache,
                                  const float* __restrict__ pk, const float* __restrict__ pv,
                                  const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
-                                 const int* __restrict__ ctx_lens, const float* __restrict__ head_scale, long long items,
+                                 const int* __restrict__ ctx_lens, const float* __restrict__ head_scale,
                                  int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E) {
-  extern __shared__ float q_lds[];  // [waves][d], q * scale * head_scale[h]
+  extern __shared__ float lds[];      // [d] q * scale * head_scale[h]; [waves][64] probabilities; [waves][dv + 2] results
+  constexpr int N = RowPiece<T>::N, COLS = kWpMaxValueDim / kWave;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const long long item = static_cast<long long>(blockIdx.x) * kWpWaves + wave;
-  const bool active = item < items;
-  const int row = active ? static_cast<int>(item / nh) : 0;
-  const int head = active ? static_cast<int>(item % nh) : 0;
-  float* qs = q_lds + wave * d;
-  if (active) {
+  const int row = blockIdx.x / nh, head = blockIdx.x % nh;
+  float* qs = lds;
+  float* ps = lds + d + wave * kWave;
+  float* merge = lds + d + kWpWaves * kWave;
+  {
     const float f = head_scale ? scale * head_scale[head] : scale;
-    for (int i = lane; i < d; i += kWave) qs[i] = load_f(q + size_t(row) * ldq + size_t(head) * d + i) * f;
+    for (int i = threadIdx.x; i < d; i += kWpWaves * kWave) qs[i] = load_f(q + size_t(row) * ldq + size_t(head) * d + i) * f;
   }
   __syncthreads();
-  if (!active) return;
-
   const int kvh = head / (nh / nkv);
   const int ctx = ctx_lens[row];
   T* orow = out + size_t(row) * ldo + size_t(head) * dv;
   if (ctx <= 0) {
-    for (int i = lane; i < dv; i += kWave) store_f(orow + i, 0.f);
+    for (int i = threadIdx.x; i < dv; i += kWpWaves * kWave) store_f(orow + i, 0.f);
     return;
   }
   const int* table = tables + size_t(row_seq[row]) * table_stride;
   const int first = (window > 0 && ctx > window) ? ctx - window : 0;
-  // blocks that end at or before position (ctx - 1) - window
-  const int blocks = (P > 0 && window > 0 && ctx - window >= P) ? (ctx - window) / P : 0;
-
-  float m = -INFINITY, l = 0.f;
-  float o[kWpMaxValueDim / kWave];
-#pragma unroll
-  for (int i = 0; i < kWpMaxValueDim / kWave; ++i) o[i] = 0.f;
-
-  for (int c0 = 0; c0 < blocks; c0 += kWave) {
-    const int b = c0 + lane;
-    const bool valid = b < blocks;
-    float s = -INFINITY;
-    int page = 0, entry = 0;
-    if (valid) {
-      const int e = b * P + P - 1, pgi = e / B;
-      page = table[pgi];
-      entry = b - (pgi * B) / P;
-      const float* kp = pk + ((size_t(page) * nkv + kvh) * E + entry) * d;
-      s = 0.f;
-      for (int i = 0; i < d; ++i) s = fmaf(qs[i], kp[i], s);
-    }
-    const float m_new = fmaxf(m, wave_max(s));
-    const float alpha = expf(m - m_new);
-    const float p = valid ? expf(s - m_new) : 0.f;
-    l = l * alpha + wave_sum(p);
-#pragma unroll
-    for (int i = 0; i < kWpMaxValueDim / kWave; ++i) o[i] *= alpha;
-    const int n = blocks - c0 < kWave ? blocks - c0 : kWave;
-    for (int j = 0; j < n; ++j) {
-      const float pj = __shfl(p, j, kWave);
-      const int page_j = __shfl(page, j, kWave), entry_j = __shfl(entry, j, kWave);
-      const float* vp = pv + ((size_t(page_j) * nkv + kvh) * E + entry_j) * dv;
-#pragma unroll
-      for (int i = 0; i < kWpMaxValueDim / kWave; ++i) {
-        const int c = lane + i * kWave;
-        if (c < dv) o[i] = fmaf(pj, vp[c], o[i]);
-      }
-    }
-    m = m_new;
-  }
-
+  const int blocks = (P > 0 && window > 0 && ctx - window >= P) ? (ctx - window) / P : 0;      // those that end at or before ctx - 1 - window
+  const int block_chunks = (blocks + kWave - 1) / kWave;
+  const int first_chunk = first / kWave, chunks = block_chunks + ((ctx - 1) / kWave - first_chunk + 1);
+  const bool wide_k = (d % N == 0) && (reinterpret_cast<uintptr_t>(kcache) % 16 == 0);
+  const bool wide_pk = (d % 4 == 0);
+  const bool wide_v = (B % N == 0) && (reinterpret_cast<uintptr_t>(vcache) % 16 == 0);
   const size_t khead = size_t(B) * d, kpage = khead * nkv;
   const size_t vhead = size_t(B) * dv, vpage = vhead * nkv;
-  for (int c0 = (first / kWave) * kWave; c0 < ctx; c0 += kWave) {
+
+  float m = -INFINITY, l = 0.f;
+  float o[COLS];
+#pragma unroll
+  for (int i = 0; i < COLS; ++i) o[i] = 0.f;
+
+  for (int c = wave; c < chunks; c += kWpWaves) {
+    const bool pooled = c < block_chunks;
+    const int c0 = pooled ? c * kWave : (first_chunk + (c - block_chunks)) * kWave;
     const int t = c0 + lane;
-    const bool valid = t >= first && t < ctx;
     float s = -INFINITY;
-    if (valid) {
-      const T* kp = kcache + size_t(table[t / B]) * kpage + kvh * khead + size_t(t % B) * d;
-      s = 0.f;
-      for (int i = 0; i < d; ++i) s = fmaf(qs[i], load_f(kp + i), s);
+    int page = 0, entry = 0;
+    bool valid;
+    if (pooled) {
+      valid = t < blocks;
+      if (valid) {
+        const int e = t * P + P - 1, pgi = e / B;
+        page = table[pgi];
+        entry = t - (pgi * B) / P;
+        s = dot_row<float>(qs, pk + ((size_t(page) * nkv + kvh) * E + entry) * d, d, wide_pk);
+      }
+    } else {
+      valid = t >= first && t < ctx;
+      if (valid) s = dot_row<T>(qs, kcache + size_t(table[t / B]) * kpage + kvh * khead + size_t(t % B) * d, d, wide_k);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float alpha = expf(m - m_new);
     const float p = valid ? expf(s - m_new) : 0.f;
     l = l * alpha + wave_sum(p);
 #pragma unroll
-    for (int i = 0; i < kWpMaxValueDim / kWave; ++i) o[i] *= alpha;
-    const int j_lo = first > c0 ? first - c0 : 0;
-    const int j_hi = ctx - c0 < kWave ? ctx - c0 : kWave;
-    for (int j = j_lo; j < j_hi; ++j) {
-      const float pj = __shfl(p, j, kWave);
-      const int tj = c0 + j;
-      const T* vp = vcache + size_t(table[tj / B]) * vpage + kvh * vhead + tj % B;  // [dim][slot]
+    for (int i = 0; i < COLS; ++i) o[i] *= alpha;
+    m = m_new;
+    __builtin_amdgcn_wave_barrier();
+    ps[lane] = p;
+    __builtin_amdgcn_wave_barrier();
+    if (pooled) {
+      const int n = blocks - c0 < kWave ? blocks - c0 : kWave;
+      for (int j = 0; j < n; ++j) {
+        const int page_j = __shfl(page, j, kWave), entry_j = __shfl(entry, j, kWave);
+        const float* vp = pv + ((size_t(page_j) * nkv + kvh) * E + entry_j) * dv;
+        const float pj = ps[j];
 #pragma unroll
-      for (int i = 0; i < kWpMaxValueDim / kWave; ++i) {
-        const int c = lane + i * kWave;
-        if (c < dv) o[i] = fmaf(pj, load_f(vp + size_t(c) * B), o[i]);
+        for (int i = 0; i < COLS; ++i) {
+          const int cc = lane + i * kWave;
+          if (cc < dv) o[i] = fmaf(pj, vp[cc], o[i]);
+        }
+      }
+    } else {
+      const int j_lo = first > c0 ? first - c0 : 0;
+      const int j_hi = ctx - c0 < kWave ? ctx - c0 : kWave;
+      if (wide_v) {
+        for (int j0 = (j_lo / N) * N; j0 < j_hi; j0 += N) {      // N tokens of one page at a time
+          const int tj = c0 + j0;
+          const T* vp = vcache + size_t(table[tj / B]) * vpage + kvh * vhead + tj % B;      // [column][slot]
+#pragma unroll
+          for (int i = 0; i < COLS; ++i) {
+            const int cc = lane + i * kWave;
+            if (cc < dv) {
+              float f[N];
+              unpack_piece(vp + size_t(cc) * B, f);
+#pragma unroll
+              for (int e = 0; e < N; ++e)
+                if (j0 + e >= j_lo && j0 + e < j_hi) o[i] = fmaf(ps[j0 + e], f[e], o[i]);      // beyond the context: stale values, never used
+            }
+          }
+        }
+      } else {
+        for (int j = j_lo; j < j_hi; ++j) {
+          const int tj = c0 + j;
+          const T* vp = vcache + size_t(table[tj / B]) * vpage + kvh * vhead + tj % B;
+          const float pj = ps[j];
+#pragma unroll
+          for (int i = 0; i < COLS; ++i) {
+            const int cc = lane + i * kWave;
+            if (cc < dv) o[i] = fmaf(pj, load_f(vp + size_t(cc) * B), o[i]);
+          }
+        }
       }
     }
-    m = m_new;
   }
+  // merge the waves' results in wave order
+  float* mine = merge + wave * (dv + 2);
 #pragma unroll
-  for (int i = 0; i < kWpMaxValueDim / kWave; ++i) {
-    const int c = lane + i * kWave;
-    if (c < dv) store_f(orow + c, o[i] / l);
+  for (int i = 0; i < COLS; ++i) {
+    const int cc = lane + i * kWave;
+    if (cc < dv) mine[cc] = o[i];
+  }
+  if (lane == 0) {
+    mine[dv] = m;
+    mine[dv + 1] = l;
+  }
+  __syncthreads();
+  float mm = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < kWpWaves; ++w) mm = fmaxf(mm, merge[w * (dv + 2) + dv]);
+  float wgt[kWpWaves], ll = 0.f;
+#pragma unroll
+  for (int w = 0; w < kWpWaves; ++w) {
+    const float mw = merge[w * (dv + 2) + dv];
+    wgt[w] = mw == -INFINITY ? 0.f : expf(mw - mm);
+    ll = fmaf(merge[w * (dv + 2) + dv + 1], wgt[w], ll);
+  }
+  for (int cc = threadIdx.x; cc < dv; cc += kWpWaves * kWave) {
+    float acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWpWaves; ++w) acc = fmaf(merge[w * (dv + 2) + cc], wgt[w], acc);
+    store_f(orow + cc, acc / ll);
   }
 }
 
@@ -279,19 +355,18 @@ int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int
   KVCM_REQUIRE(ldq >= nh * d && ldo >= nh * dv, "attention_window_pool: row strides too small");
   KVCM_REQUIRE(window >= 0 && P >= 0, "attention_window_pool: negative window or block");
   KVCM_REQUIRE(P == 0 || (pk && pv && E == (B + P - 1) / P), "attention_window_pool: pooled blocks need their entries");
-  const long long items = static_cast<long long>(T) * nh;
-  const long long blocks = (items + kWpWaves - 1) / kWpWaves;
+  const long long blocks = static_cast<long long>(T) * nh;
   KVCM_REQUIRE(blocks < (1ll << 31), "attention_window_pool: too many rows");
-  const size_t lds = sizeof(float) * kWpWaves * d;
+  const size_t lds = sizeof(float) * (d + kWpWaves * kWave + kWpWaves * (dv + 2));
   if (dtype == kF32)
     attention_window_pool_kernel<float><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const float*>(q), ldq, static_cast<float*>(out), ldo, static_cast<const float*>(kcache),
-        static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, items, nh, nkv, d, dv,
+        static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, nh, nkv, d, dv,
         B, scale, window, P, E);
   else if (dtype == kBF16)
     attention_window_pool_kernel<bf16_t><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const bf16_t*>(q), ldq, static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(kcache),
-        static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, items, nh, nkv, d, dv,
+        static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, nh, nkv, d, dv,
         B, scale, window, P, E);
   else KVCM_REQUIRE(false, "attention_window_pool: unknown dtype %d", dtype);
   return launch_status("attention_window_pool");

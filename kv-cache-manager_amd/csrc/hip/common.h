@@ -73,6 +73,24 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Sum over aligned groups of G lanes (a power of two); every lane of a group gets the result.  Up to 16 lanes the
+// partners come by data-parallel-primitive moves inside a row of 16 (a few cycles each: lane ^ 1, lane ^ 2, then the
+// mirrored half and the mirrored row, whose lanes hold the other half's sum already); beyond that by shuffles.
+template <int CTRL>
+__device__ __forceinline__ float dpp_take(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+  if constexpr (G >= 2) v += dpp_take<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+  if constexpr (G >= 4) v += dpp_take<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+  if constexpr (G >= 8) v += dpp_take<0x141>(v);      // row_half_mirror
+  if constexpr (G >= 16) v += dpp_take<0x140>(v);     // row_mirror
+  if constexpr (G >= 32) v += __shfl_xor(v, 16, kWave);
+  if constexpr (G >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
 // Sum over a block of THREADS threads (a multiple of 64); every thread gets the result.  The
 // order of additions depends on THREADS only.
 template <int THREADS>

@@ -10,11 +10,11 @@
 //
 // Two launches.  The first turns the projections of every row into (w, a * u, u), in parallel over rows
 // (the second step of the decay's projection included).
-// The second walks each sequence's run token by token: a workgroup per (sequence, head), a thread per
-// value column j that keeps S[:, j] in registers; per token it needs u^T S[:, j] (a sum over its own
-// registers), updates its column and sums o_j: no thread needs another's column.  The per-token vectors
-// (r, k, w, a*u, u) are staged through LDS a few tokens at a time.  A run that starts at position 0
-// starts from zero without reading its slot.  Tokens are taken one by one in prompts and in decoding.
+// The second walks each sequence's run token by token: a value column j of S needs u^T S[:, j], updates itself
+// and sums o_j, and needs no other column, so columns are spread over lanes and workgroups.  The per-token
+// vectors (r, k, w, a*u, u, v) are staged through LDS a few tokens at a time, the next tokens' values
+// requested before the current ones are computed.  A run that starts at position 0 starts from zero
+// without reading its slot.  Tokens are taken one by one in prompts and in decoding.
 #include "common.h"
 #include "kvcm_hip.h"
 
@@ -60,73 +60,111 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-template <int DKP>
+// The state of one head is dk x dv.  A workgroup of 256 threads owns 256 / G value columns of one head of one
+// sequence; the key dimension of a column is spread over G lanes (IPT = DKP / G entries each, DKP: dk padded
+// with zeros), so a token costs a lane IPT multiply-adds for u^T S, a sum across its G lanes, 3 IPT
+// multiply-adds for the update, IPT for o and another sum across the lanes.
+template <int DKP, int G>
 __global__ void __launch_bounds__(256)
     delta_scan_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
                       const float* __restrict__ v, int ldv, const float* __restrict__ w, const float* __restrict__ au,
                       const float* __restrict__ u, float* __restrict__ o, int ldo, float* __restrict__ state,
                       const int* __restrict__ run_start, const int* __restrict__ seq_start,
-                      const int* __restrict__ state_slots, int heads, int dk, int dv) {
-  __shared__ float tile[kDeltaTile][5][DKP];      // r, k, w, a*u, u of the staged tokens (zero beyond dk)
-  const int s = blockIdx.y, head = blockIdx.x;
-  const int j = threadIdx.x;
+                      const int* __restrict__ state_slots, int heads, int dk, int dv, int col_blocks) {
+  constexpr int IPT = DKP / G, CB = 256 / G, W = 5 * DKP + CB;
+  constexpr int PF = (kDeltaTile * W + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float tile[kDeltaTile][W];      // per token: r, k, w, a*u, u (zero beyond dk), v of these columns
+  const int s = blockIdx.y, head = blockIdx.x / col_blocks, cb = blockIdx.x % col_blocks;
+  const int g = threadIdx.x % G, j = cb * CB + threadIdx.x / G;
   const int r0 = run_start[s], r1 = run_start[s + 1];
   const int slot = state_slots[s];
   if (r1 <= r0) return;
   const size_t D = size_t(heads) * dk;
+  const bool owns = j < dv;
   if (slot < 0) {
-    if (j < dv)
+    if (owns && g == 0)
       for (int row = r0; row < r1; ++row) o[size_t(row) * ldo + size_t(head) * dv + j] = 0.f;
     return;
   }
-  float* st = state + ((size_t(slot) * heads + head) * dk) * dv + j;      // [slot][head][i][j]
+  float* st = state + ((size_t(slot) * heads + head) * dk) * dv + (owns ? j : 0);      // [slot][head][i][j]
   const bool fresh = seq_start[s] == 0;
-  float S[DKP];
+  float S[IPT];
 #pragma unroll
-  for (int i = 0; i < DKP; ++i) S[i] = (i < dk && j < dv && !fresh) ? st[size_t(i) * dv] : 0.f;
-
-  for (int t0 = r0; t0 < r1; t0 += kDeltaTile) {
-    const int nt = r1 - t0 < kDeltaTile ? r1 - t0 : kDeltaTile;
-    __syncthreads();
-    for (int e = threadIdx.x; e < nt * 5 * DKP; e += blockDim.x) {
-      const int t = e / (5 * DKP), which = (e / DKP) % 5, i = e % DKP;
+  for (int il = 0; il < IPT; ++il) {
+    const int i = g * IPT + il;
+    S[il] = (i < dk && owns && !fresh) ? st[size_t(i) * dv] : 0.f;
+  }
+  float pf[PF];
+  auto request = [&](int t0) {      // the staged values of the tokens t0 .. t0 + tile - 1, into registers
+#pragma unroll
+    for (int q = 0; q < PF; ++q) {
+      const int e = threadIdx.x + q * 256;
+      const int t = e / W, off = e % W;
       const int row = t0 + t;
       float val = 0.f;
-      if (i < dk) {
-        const size_t col = size_t(head) * dk + i;
-        if (which == 0) val = r[size_t(row) * ldr + col];
-        else if (which == 1) val = k[size_t(row) * ldk + col];
-        else if (which == 2) val = w[size_t(row) * D + col];
-        else if (which == 3) val = au[size_t(row) * D + col];
-        else val = u[size_t(row) * D + col];
+      if (t < kDeltaTile && row < r1) {
+        if (off < 5 * DKP) {
+          const int which = off / DKP, i = off % DKP;
+          if (i < dk) {
+            const size_t col = size_t(head) * dk + i;
+            if (which == 0) val = r[size_t(row) * ldr + col];
+            else if (which == 1) val = k[size_t(row) * ldk + col];
+            else if (which == 2) val = w[size_t(row) * D + col];
+            else if (which == 3) val = au[size_t(row) * D + col];
+            else val = u[size_t(row) * D + col];
+          }
+        } else {
+          const int jj = cb * CB + (off - 5 * DKP);
+          if (jj < dv) val = v[size_t(row) * ldv + size_t(head) * dv + jj];
+        }
       }
-      tile[t][which][i] = val;
+      pf[q] = val;
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int q = 0; q < PF; ++q) {
+      const int e = threadIdx.x + q * 256;
+      if (e < kDeltaTile * W) tile[e / W][e % W] = pf[q];
+    }
+  };
+  request(r0);
+  stage();
+  __syncthreads();
+  for (int t0 = r0; t0 < r1; t0 += kDeltaTile) {
+    const int nt = r1 - t0 < kDeltaTile ? r1 - t0 : kDeltaTile;
+    const bool more = t0 + kDeltaTile < r1;
+    if (more) request(t0 + kDeltaTile);
+    for (int t = 0; t < nt; ++t) {
+      const float* tv = tile[t];
+      const float vj = tv[5 * DKP + threadIdx.x / G];
+      float sa = 0.f;
+#pragma unroll
+      for (int il = 0; il < IPT; ++il) sa = fmaf(tv[4 * DKP + g * IPT + il], S[il], sa);
+      sa = group_sum<G>(sa);
+      float acc = 0.f;
+#pragma unroll
+      for (int il = 0; il < IPT; ++il) {
+        const int i = g * IPT + il;
+        float sn = tv[2 * DKP + i] * S[il];
+        sn = fmaf(-tv[3 * DKP + i], sa, sn);
+        sn = fmaf(tv[DKP + i], vj, sn);
+        S[il] = sn;
+        acc = fmaf(sn, tv[i], acc);
+      }
+      acc = group_sum<G>(acc);
+      if (owns && g == 0) o[size_t(t0 + t) * ldo + size_t(head) * dv + j] = acc;
     }
     __syncthreads();
-    if (j < dv) {
-      for (int t = 0; t < nt; ++t) {
-        const int row = t0 + t;
-        const float vj = v[size_t(row) * ldv + size_t(head) * dv + j];
-        float sa = 0.f;
-#pragma unroll
-        for (int i = 0; i < DKP; ++i) sa = fmaf(tile[t][4][i], S[i], sa);
-        float acc = 0.f;
-#pragma unroll
-        for (int i = 0; i < DKP; ++i) {
-          float sn = tile[t][2][i] * S[i];
-          sn = fmaf(-tile[t][3][i], sa, sn);
-          sn = fmaf(tile[t][1][i], vj, sn);
-          S[i] = sn;
-          acc = fmaf(sn, tile[t][0][i], acc);
-        }
-        o[size_t(row) * ldo + size_t(head) * dv + j] = acc;
-      }
-    }
+    if (more) stage();
+    __syncthreads();
   }
-  if (j < dv) {
+  if (owns) {
 #pragma unroll
-    for (int i = 0; i < DKP; ++i)
-      if (i < dk) st[size_t(i) * dv] = S[i];
+    for (int il = 0; il < IPT; ++il) {
+      const int i = g * IPT + il;
+      if (i < dk) st[size_t(i) * dv] = S[il];
+    }
   }
 }
 
@@ -160,18 +198,21 @@ int kvcm_delta_scan(const float* r, int ldr, const float* k, int ldk, const floa
                     const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s) {
   if (S == 0) return 0;
   KVCM_REQUIRE(S > 0 && heads > 0 && dk > 0 && dv > 0, "delta_scan: bad sizes S=%d heads=%d dk=%d dv=%d", S, heads, dk, dv);
-  KVCM_REQUIRE(dk <= 128 && dv <= 256, "delta_scan: key size %d / value size %d are not supported (up to 128 / 256)", dk, dv);
+  KVCM_REQUIRE(dk <= 128, "delta_scan: a key size of %d is not supported (up to 128)", dk);
+  KVCM_REQUIRE(static_cast<long long>(heads) * ((dv + 31) / 32) < (1ll << 31), "delta_scan: too many heads");
   KVCM_REQUIRE(S <= 65535, "delta_scan: too many sequences for one launch (%d)", S);
   KVCM_REQUIRE(ldr >= heads * dk && ldk >= heads * dk && ldv >= heads * dv && ldo >= heads * dv, "delta_scan: row strides too small");
-  const dim3 grid(heads, S);
-  const int threads = ((dv + kWave - 1) / kWave) * kWave;
-#define KVCM_DELTA(DKP)                                                                                              \
-  delta_scan_kernel<DKP><<<grid, threads, 0, s>>>(r, ldr, k, ldk, v, ldv, w, au, u, o, ldo, state, run_start, seq_start, \
-                                                  state_slots, heads, dk, dv)
-  if (dk <= 16) KVCM_DELTA(16);
-  else if (dk <= 32) KVCM_DELTA(32);
-  else if (dk <= 64) KVCM_DELTA(64);
-  else KVCM_DELTA(128);
+#define KVCM_DELTA(DKP, G)                                                                                            \
+  {                                                                                                                    \
+    const int col_blocks = (dv + 256 / G - 1) / (256 / G);                                                             \
+    delta_scan_kernel<DKP, G><<<dim3(heads * col_blocks, S), 256, 0, s>>>(r, ldr, k, ldk, v, ldv, w, au, u, o, ldo, state, \
+                                                                          run_start, seq_start, state_slots, heads, dk, dv, \
+                                                                          col_blocks);                                  \
+  }
+  if (dk <= 16) KVCM_DELTA(16, 2)
+  else if (dk <= 32) KVCM_DELTA(32, 4)
+  else if (dk <= 64) KVCM_DELTA(64, 8)
+  else KVCM_DELTA(128, 8)
 #undef KVCM_DELTA
   return launch_status("delta_scan");
 }

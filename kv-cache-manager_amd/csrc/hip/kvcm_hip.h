@@ -146,6 +146,7 @@ int kvcm_probe_phases(const void* weights, const long long* phase_bytes, int pha
 int kvcm_embed_scaled(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, float factor,
                       hipStream_t s);
 int kvcm_gated_act(const float* gate_up, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s);
+int kvcm_widen(const void* in, float* out, long long n, hipStream_t s);      // contiguous bfloat16 -> 32-bit
 // (norm_chain.hip) 32-bit RMS norms chained along a row: two branches combined, normed, added to the stream, the
 // stream normed again; the norm of every head with a weight and a sigmoid gate
 int kvcm_rmsnorm_chain(float* x, const float* a, const float* b, const float* wa, const float* wb, float combine,
@@ -172,6 +173,13 @@ int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int
                                const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
                                const int* ctx_lens, const float* head_scale, int T, int nh, int nkv, int d, int dv, int B,
                                float scale, int window, int P, int E, hipStream_t s);
+// (attention_window_pool_tiles.hip) the same attention for runs of consecutive positions, on the matrix cores (bfloat16)
+int kvcm_attention_window_pool_tiles_supported(int d, int dv, int B);
+int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
+                                     const float* pk, const float* pv, const int* tables, int table_stride,
+                                     const int* run_start, const int* seq_start, const float* head_scale, int S, int max_run,
+                                     int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
+                                     hipStream_t s);
 // (selective_scan.hip, delta_rule.hip) recurrences with a 32-bit state per sequence
 int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
                         const float* bc, int ldbc, int off_b, int off_c, const float* a_log, const float* dskip,

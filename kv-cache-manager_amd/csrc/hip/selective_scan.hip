@@ -6,18 +6,22 @@
 //   y_c = sum_n S[c, n] * C_n + D_c * x_c;   out_c = y_c * silu(z_c)
 //
 // Everything of the recurrence is 32-bit: the state, the step size with its softplus, the decay's
-// exponential, the sums.  A thread owns one channel of one sequence, keeps that channel's row of the
-// state and of A in registers and walks the run's tokens in order; B and C of a token are the same for
-// every channel, so a wave's loads of them are broadcasts.  A run that starts at position 0 starts
-// from zero without reading its slot; the state after the run's last token goes back to the slot.
-// Tokens are taken one by one in both prompts and decoding, so a position's result does not depend on
-// how the prompt was cut.
+// exponential, the sums.  The states of a channel are spread over LPC lanes (a power of two, up to a whole
+// wave; NPL states a lane beyond that), so that a wave of 64 lanes walks 64 / LPC channels: the run's
+// tokens are taken in order, one exponential and two multiply-adds a lane and token, and the sum over a
+// channel's states crosses its lanes in a fixed tree.  What a token brings (its step size, input, gate, B
+// and C) does not depend on the state: it is requested a few tokens ahead, so that the walk waits for
+// arithmetic and not for memory.  A run that starts at position 0 starts from zero without reading its
+// slot; the state after the run's last token goes back to the slot.  Tokens are taken one by one in both
+// prompts and decoding, so a position's result does not depend on how the prompt was cut.
 #include "common.h"
 #include "kvcm_hip.h"
 
 namespace kvcm {
 
-template <class T, int NP>
+constexpr int kScanAhead = 4;      // tokens whose inputs are on their way while the ones before are computed
+
+template <class T, int LPC, int NPL>
 __global__ void __launch_bounds__(kWave)
     selective_scan_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ dt_lin, int lddt,
                           const float* __restrict__ dt_bias, const float* __restrict__ bc, int ldbc, int off_b, int off_c,
@@ -25,46 +29,88 @@ __global__ void __launch_bounds__(kWave)
                           int ldz, T* __restrict__ out, int ldo, float* __restrict__ state,
                           const int* __restrict__ run_start, const int* __restrict__ seq_start,
                           const int* __restrict__ state_slots, int C, int N) {
+  constexpr int U = kScanAhead;
   const int s = blockIdx.y;
-  const int c = blockIdx.x * kWave + threadIdx.x;
+  const int sub = threadIdx.x % LPC;
+  const int c_real = blockIdx.x * (kWave / LPC) + threadIdx.x / LPC;
+  const bool owns = c_real < C;
+  const int c = owns ? c_real : C - 1;      // lanes beyond the last channel walk along (the sums cross lanes) and store nothing
   const int r0 = run_start[s], r1 = run_start[s + 1];
   const int slot = state_slots[s];
-  if (c >= C || r1 <= r0) return;
+  if (r1 <= r0) return;
   if (slot < 0) {      // a padding sequence: its rows carry nothing
-    for (int r = r0; r < r1; ++r) store_f(out + size_t(r) * ldo + c, 0.f);
+    if (owns && sub == 0)
+      for (int r = r0; r < r1; ++r) store_f(out + size_t(r) * ldo + c, 0.f);
     return;
   }
   float* st = state + (size_t(slot) * C + c) * N;
   const bool fresh = seq_start[s] == 0;
-  float S[NP], A[NP];
+  float S[NPL], A[NPL];
+  int nidx[NPL];
+  bool has[NPL];
 #pragma unroll
-  for (int n = 0; n < NP; ++n) {
-    A[n] = n < N ? -expf(a_log[size_t(c) * N + n]) : 0.f;
-    S[n] = (n < N && !fresh) ? st[n] : 0.f;
+  for (int k = 0; k < NPL; ++k) {
+    const int n = sub + k * LPC;
+    has[k] = n < N;
+    nidx[k] = has[k] ? n : N - 1;
+    A[k] = has[k] ? -expf(a_log[size_t(c) * N + nidx[k]]) : 0.f;
+    S[k] = (has[k] && !fresh) ? st[nidx[k]] : 0.f;
   }
   const float db = dt_bias ? dt_bias[c] : 0.f, dk = dskip[c];
-  for (int r = r0; r < r1; ++r) {
-    const float v = dt_lin[size_t(r) * lddt + c] + db;
-    const float dt = v > 20.f ? v : log1pf(expf(v));
-    const float xv = load_f(x + size_t(r) * ldx + c);
-    const float dx = dt * xv;
-    const float* brow = bc + size_t(r) * ldbc + off_b;
-    const float* crow = bc + size_t(r) * ldbc + off_c;
-    float y = 0.f;
+
+  float dtv[2][U], xv[2][U], zv[2][U], bv[2][U][NPL], cv[2][U][NPL];
+  auto request = [&](int first, int into) {
 #pragma unroll
-    for (int n = 0; n < NP; ++n) {
-      if (n < N) {
-        S[n] = fmaf(expf(dt * A[n]), S[n], dx * brow[n]);
-        y = fmaf(S[n], crow[n], y);
+    for (int u = 0; u < U; ++u) {
+      const int r = first + u < r1 ? first + u : r1 - 1;
+      dtv[into][u] = dt_lin[size_t(r) * lddt + c];
+      xv[into][u] = load_f(x + size_t(r) * ldx + c);
+      zv[into][u] = z[size_t(r) * ldz + c];
+#pragma unroll
+      for (int k = 0; k < NPL; ++k) {
+        bv[into][u][k] = bc[size_t(r) * ldbc + off_b + nidx[k]];
+        cv[into][u][k] = bc[size_t(r) * ldbc + off_c + nidx[k]];
       }
     }
-    y = fmaf(dk, xv, y);
-    const float zv = z[size_t(r) * ldz + c];
-    store_f(out + size_t(r) * ldo + c, y * (zv / (1.0f + expf(-zv))));
-  }
+  };
+  auto walk = [&](int first, int from) {
 #pragma unroll
-  for (int n = 0; n < NP; ++n)
-    if (n < N) st[n] = S[n];
+    for (int u = 0; u < U; ++u) {
+      const int r = first + u;
+      if (r < r1) {
+        const float v = dtv[from][u] + db;
+        const float dt = v > 20.f ? v : log1pf(expf(v));
+        const float dx = dt * xv[from][u];
+        float y = 0.f;
+#pragma unroll
+        for (int k = 0; k < NPL; ++k) {
+          const float sn = fmaf(expf(dt * A[k]), S[k], dx * bv[from][u][k]);
+          S[k] = has[k] ? sn : 0.f;
+          y = fmaf(S[k], cv[from][u][k], y);
+        }
+        y = group_sum<LPC>(y);
+        if (owns && sub == 0) {
+          y = fmaf(dk, xv[from][u], y);
+          const float zz = zv[from][u];
+          store_f(out + size_t(r) * ldo + c, y * (zz / (1.0f + expf(-zz))));
+        }
+      }
+    }
+  };
+  request(r0, 0);
+  for (int r = r0; r < r1; r += 2 * U) {
+    if (r + U < r1) request(r + U, 1);
+    walk(r, 0);
+    if (r + U < r1) {
+      if (r + 2 * U < r1) request(r + 2 * U, 0);
+      walk(r + U, 1);
+    }
+  }
+  if (owns) {
+#pragma unroll
+    for (int k = 0; k < NPL; ++k)
+      if (has[k]) st[nidx[k]] = S[k];
+  }
 }
 
 template <class T>
@@ -72,16 +118,18 @@ int launch_scan(const void* x, int ldx, const float* dt_lin, int lddt, const flo
                 int off_b, int off_c, const float* a_log, const float* dskip, const float* z, int ldz, void* out, int ldo,
                 float* state, const int* run_start, const int* seq_start, const int* state_slots, int S, int C, int N,
                 hipStream_t s) {
-  const dim3 grid((C + kWave - 1) / kWave, S);
-#define KVCM_SCAN(NP)                                                                                                  \
-  selective_scan_kernel<T, NP><<<grid, kWave, 0, s>>>(static_cast<const T*>(x), ldx, dt_lin, lddt, dt_bias, bc, ldbc, off_b, \
-                                                      off_c, a_log, dskip, z, ldz, static_cast<T*>(out), ldo, state,   \
-                                                      run_start, seq_start, state_slots, C, N)
-  if (N <= 8) KVCM_SCAN(8);
-  else if (N <= 16) KVCM_SCAN(16);
-  else if (N <= 32) KVCM_SCAN(32);
-  else if (N <= 64) KVCM_SCAN(64);
-  else KVCM_SCAN(128);
+#define KVCM_SCAN(LPC, NPL)                                                                                             \
+  selective_scan_kernel<T, LPC, NPL><<<dim3((C + kWave / LPC - 1) / (kWave / LPC), S), kWave, 0, s>>>(                   \
+      static_cast<const T*>(x), ldx, dt_lin, lddt, dt_bias, bc, ldbc, off_b, off_c, a_log, dskip, z, ldz,               \
+      static_cast<T*>(out), ldo, state, run_start, seq_start, state_slots, C, N)
+  if (N <= 1) KVCM_SCAN(1, 1);
+  else if (N <= 2) KVCM_SCAN(2, 1);
+  else if (N <= 4) KVCM_SCAN(4, 1);
+  else if (N <= 8) KVCM_SCAN(8, 1);
+  else if (N <= 16) KVCM_SCAN(16, 1);
+  else if (N <= 32) KVCM_SCAN(32, 1);
+  else if (N <= 64) KVCM_SCAN(64, 1);
+  else KVCM_SCAN(64, 2);
 #undef KVCM_SCAN
   return launch_status("selective_scan");
 }

@@ -92,6 +92,7 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_sample),
     KVCM_ENTRY(kvcm_embed_scaled),
     KVCM_ENTRY(kvcm_gated_act),
+    KVCM_ENTRY(kvcm_widen),
     KVCM_ENTRY(kvcm_rmsnorm_chain),
     KVCM_ENTRY(kvcm_head_norm_gate),
     KVCM_ENTRY(kvcm_short_conv),
@@ -100,6 +101,7 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_rotate_store),
     KVCM_ENTRY(kvcm_pool_update),
     KVCM_ENTRY(kvcm_attention_window_pool),
+    KVCM_ENTRY(kvcm_attention_window_pool_tiles),
     KVCM_ENTRY(kvcm_selective_scan),
     KVCM_ENTRY(kvcm_delta_prepare),
     KVCM_ENTRY(kvcm_delta_scan),

@@ -87,6 +87,7 @@ def _declare(lib):
     fn("kvcm_gemm8_residual_norm", vp, i, vp, i, i, i, i, vp, vp, i, vp, vp, vp)
     fn("kvcm_embed_scaled", vp, vp, i, vp, i, i, i, f, vp)
     fn("kvcm_gated_act", vp, i, vp, i, i, i, i, i, vp)
+    fn("kvcm_widen", vp, vp, C.c_longlong, vp)
     fn("kvcm_rmsnorm_chain", vp, vp, vp, vp, vp, f, vp, vp, vp, vp, i, i, i, f, vp)
     fn("kvcm_head_norm_gate", vp, i, vp, i, vp, vp, i, i, i, i, i, f, vp)
     fn("kvcm_short_conv", vp, i, vp, vp, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, vp)
@@ -95,6 +96,8 @@ def _declare(lib):
     fn("kvcm_rotate_store", vp, i, vp, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_pool_update", vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp)
+    fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
+    fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, vp)
     fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_delta_prepare", vp, i, vp, i, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_delta_scan", vp, i, vp, i, vp, i, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, vp)
@@ -942,6 +945,20 @@ def gated_act(gate_up, out, activation):
           GATE_ACTIVATIONS[activation], _stream())
 
 
+def widen(x, out):
+    """out (float32) = x (bfloat16), both contiguous and of one shape."""
+    _dev(x, out)
+    _need(x.dtype == torch.bfloat16 and out.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
+          and x.shape == out.shape, "widen takes a contiguous bfloat16 tensor and a float32 one of the same shape")
+    _call("kvcm_widen", _ptr(x), _ptr(out), x.numel(), _stream())
+    return out
+
+
+def library_takes(M, N, K):
+    """Does a bfloat16 product of this shape go to the vendor library (when its result is bfloat16)?"""
+    return bool(_library_takes(M, N, K))
+
+
 class NormedBranches:
     """A sublayer's output that is still to be normed and added to the residual stream:
     x += n(m) * w_post with m = a, or m = combine * (n(a) * wa + n(b) * wb) for two branches side by side
@@ -1112,6 +1129,30 @@ def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, 
     _call("kvcm_attention_window_pool", _ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
           _ptr(pk), _ptr(pv), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), _ptr(head_scale), T, nh, nkv, d, dv,
           B, float(scale), int(window), int(P), E, _stream())
+
+
+def attention_window_pool_tiles_supported(d, dv, dtype, block_size):
+    """Does the matrix-core kernel for runs of consecutive positions take this head shape?"""
+    return dtype == torch.bfloat16 and bool(lib().kvcm_attention_window_pool_tiles_supported(d, dv, block_size))
+
+
+def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_stride, run_start, seq_start, num_seqs, max_run,
+                                nh, nkv, d, dv, scale, window, P, head_scale=None):
+    """``attention_window_pool`` for steps whose sequences run several consecutive positions: 64 rows of a run and one
+    head per workgroup on the matrix cores (bfloat16 only).  Every row of every run is computed, single rows too."""
+    _dev(q, out, kcache, vcache, tables, run_start, seq_start)
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    _need(q.dtype == out.dtype == kcache.dtype == torch.bfloat16, "the tiled attention takes bfloat16 operands")
+    _need(q.shape[1] >= nh * d and out.shape[1] >= nh * dv, "attention rows are too short for the head layout")
+    B, E = _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P)
+    _f32(head_scale, "head_scale", nh)
+    _i32(run_start, "run_start", num_seqs + 1)
+    _i32(seq_start, "seq_start", num_seqs)
+    _i32(tables, "tables")
+    _call("kvcm_attention_window_pool_tiles", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache), _ptr(pk),
+          _ptr(pv), _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), _ptr(head_scale), num_seqs, max_run, nh, nkv,
+          d, dv, B, float(scale), int(window), int(P), E, _stream())
 
 
 def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, state, step):

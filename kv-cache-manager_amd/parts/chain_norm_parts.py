@@ -16,6 +16,19 @@ def f32_params(tensors):
     return {k: v.float().contiguous() for k, v in tensors.items()}
 
 
+def linear32(ctx, step, x, w, name, exact=False):
+    """x @ w^T as 32-bit rows for a consumer that computes in 32-bit.  The products of this package write their
+    32-bit sums as they are.  A many-row product that the vendor library would take runs there with a bfloat16
+    result that is widened afterwards (the library's kernels are several times faster at those shapes), unless
+    ``exact``: what enters a recurrence keeps its 32-bit sums at every row count."""
+    ops = ctx.ops
+    M, N, K = x.shape[0], w.shape[0], w.shape[1]
+    if not exact and x.dtype == torch.bfloat16 and ops.library_takes(M, N, K):
+        half = _linear(ctx, step, x, w, name + "_h")
+        return ops.widen(half, step.ws(name, (M, N), torch.float32))
+    return _linear(ctx, step, x, w, name, dtype=torch.float32)
+
+
 class BranchPair:
     """Two sublayer outputs side by side, still to be combined as combine * (n(a) * wa + n(b) * wb)
     (n: division by the root mean square): what a mixer of two halves hands to the arrangement, which
@@ -113,7 +126,7 @@ class GatedFeedForward(FeedForward):
 
     def forward(self, step, h):
         I, ops = self.params["intermediate_size"], self.ctx.ops
-        gu = _linear(self.ctx, step, h, self.w["w_gate_up"], "gated_gate_up", dtype=torch.float32)
+        gu = linear32(self.ctx, step, h, self.w["w_gate_up"], "gated_gate_up")
         act = step.ws("gated_act", (step.rows, I))
         ops.gated_act(gu, act, self.params.get("activation", "silu"))
-        return _linear(self.ctx, step, act, self.w["w_down"], "gated_out", dtype=torch.float32)
+        return linear32(self.ctx, step, act, self.w["w_down"], "gated_out")

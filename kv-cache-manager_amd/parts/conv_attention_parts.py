@@ -7,7 +7,7 @@ import torch
 
 from ..registry import MIXERS, POSITIONS
 from .base import KVCacheNeed, Mixer, ParamSpec, PartSpec, PositionEncoding, StateNeed
-from .chain_norm_parts import BranchPair, f32_params
+from .chain_norm_parts import BranchPair, f32_params, linear32
 from .llama_parts import _linear
 
 
@@ -93,7 +93,7 @@ class ConvWindowPoolAttention(Mixer):
         pool = p["pool"] if p["window"] > 0 else 0
         pk, pv = (self.cache.pooled_k(self.cache_index), self.cache.pooled_v(self.cache_index)) if pool else (None, None)
         T, K = step.rows, p["conv"]
-        proj = _linear(self.ctx, step, h, w["w_qkv"], "cwp_proj", dtype=torch.float32)
+        proj = linear32(self.ctx, step, h, w["w_qkv"], "cwp_proj")
         mixed = step.ws("cwp_conv", (T, self.channels), torch.float32)
         conv_state = self.caches["conv"][0].slots(self.caches["conv"][1]) if K > 1 else None
         ops.short_conv(proj, w["conv"], mixed, step, conv_state, bias_in=w["bias"])
@@ -106,9 +106,15 @@ class ConvWindowPoolAttention(Mixer):
             ops.pool_update(kc, vc, pk, pv, step.tables(g), step.table_stride(g), step.row_seq, step.positions, slots,
                             self.nkv, self.d, self.dv, pool, T)
         attn = step.ws("cwp_attn", (T, self.nh * self.dv))
+        if step.max_run > 1 and ops.attention_window_pool_tiles_supported(self.d, self.dv, attn.dtype, kc.shape[2]):
+            # runs of consecutive positions: 64 rows of a run share every staged key, on the matrix cores
+            ops.attention_window_pool_tiles(q, attn, kc, vc, pk, pv, step.tables(g), step.table_stride(g), step.run_start,
+                                            step.seq_start, step.seqs, step.max_run, self.nh, self.nkv, self.d, self.dv,
+                                            p["scale"], p["window"], pool, head_scale=w["temp"])
+            return linear32(self.ctx, step, attn, w["w_o"], "cwp_out")
         ops.attention_window_pool(q, attn, kc, vc, pk, pv, step.tables(g), step.table_stride(g), step.row_seq, step.ctx_lens,
                                   self.nh, self.nkv, self.d, self.dv, p["scale"], p["window"], pool, head_scale=w["temp"], rows=T)
-        return _linear(self.ctx, step, attn, w["w_o"], "cwp_out", dtype=torch.float32)
+        return linear32(self.ctx, step, attn, w["w_o"], "cwp_out")
 
 
 @MIXERS.register("parallel_mixers")

@@ -7,7 +7,7 @@ import torch
 
 from ..registry import MIXERS
 from .base import Mixer, ParamSpec, StateNeed
-from .chain_norm_parts import f32_params
+from .chain_norm_parts import f32_params, linear32
 from .llama_parts import _linear
 
 _SMALL = ("conv", "conv_bias", "dt_bias", "a_log", "d_skip", "a_bias", "w0", "w2", "norm")
@@ -59,7 +59,7 @@ class SelectiveScanMixer(_StatefulMixer):
     def forward(self, step, h):
         ops, p, w = self.ctx.ops, self.params, self.w
         C, N, R, K = p["inner"], p["state"], p["dt_rank"], p["conv"]
-        xz = _linear(self.ctx, step, h, w["w_in"], "scan_xz", dtype=torch.float32)
+        xz = linear32(self.ctx, step, h, w["w_in"], "scan_xz")
         conv_state = self.state("conv") if K > 1 else None
         x = step.ws("scan_x", (step.rows, C))
         ops.short_conv(xz, w["conv"], x, step, conv_state, bias_out=w["conv_bias"], activation="silu")
@@ -70,7 +70,7 @@ class SelectiveScanMixer(_StatefulMixer):
         dt = _linear(self.ctx, step, low, w["w_dt"], "scan_dt", dtype=torch.float32)
         y = step.ws("scan_y", (step.rows, C))
         ops.selective_scan(x, dt, w["dt_bias"], bc, 0, N, w["a_log"], w["d_skip"], xz[:, C:], y, self.state("scan"), step)
-        return _linear(self.ctx, step, y, w["w_o"], "scan_out", dtype=torch.float32)
+        return linear32(self.ctx, step, y, w["w_o"], "scan_out")
 
 
 @MIXERS.register("general_delta")
@@ -122,4 +122,4 @@ class GeneralDeltaMixer(_StatefulMixer):
         ops.delta_scan(r, k, v, decay, au, u, o, self.state("delta"), step, heads, d, d)
         gated = step.ws("delta_gated", (T, D))
         ops.head_norm_gate(o, g, w["norm"], gated, heads, d, p["eps"])
-        return _linear(self.ctx, step, gated, w["w_o"], "delta_out", dtype=torch.float32)
+        return linear32(self.ctx, step, gated, w["w_o"], "delta_out")
