@@ -95,30 +95,28 @@ __global__ void __launch_bounds__(256)
     S[il] = (i < dk && owns && !fresh) ? st[size_t(i) * dv] : 0.f;
   }
   float pf[PF];
+  // (loads are unconditional, from clamped places, and masked afterwards: a branch around a load would make every
+  // one of them wait for the one before)
   auto request = [&](int t0) {      // the staged values of the tokens t0 .. t0 + tile - 1, into registers
 #pragma unroll
     for (int q = 0; q < PF; ++q) {
       const int e = threadIdx.x + q * 256;
       const int t = e / W, off = e % W;
-      const int row = t0 + t;
-      float val = 0.f;
-      if (t < kDeltaTile && row < r1) {
-        if (off < 5 * DKP) {
-          const int which = off / DKP, i = off % DKP;
-          if (i < dk) {
-            const size_t col = size_t(head) * dk + i;
-            if (which == 0) val = r[size_t(row) * ldr + col];
-            else if (which == 1) val = k[size_t(row) * ldk + col];
-            else if (which == 2) val = w[size_t(row) * D + col];
-            else if (which == 3) val = au[size_t(row) * D + col];
-            else val = u[size_t(row) * D + col];
-          }
-        } else {
-          const int jj = cb * CB + (off - 5 * DKP);
-          if (jj < dv) val = v[size_t(row) * ldv + size_t(head) * dv + jj];
-        }
-      }
-      pf[q] = val;
+      const int row = t0 + t < r1 ? t0 + t : r1 - 1;
+      const bool vector = off < 5 * DKP;
+      const int which = off / DKP, i = off % DKP;
+      const int jj = cb * CB + (off - 5 * DKP);
+      const bool ok = t < kDeltaTile && t0 + t < r1 && (vector ? i < dk : jj < dv);
+      const size_t col = size_t(head) * dk + (i < dk ? i : dk - 1);
+      const size_t vcol = size_t(head) * dv + ((jj >= 0 && jj < dv) ? jj : 0);
+      const float* src = !vector     ? v + size_t(row) * ldv + vcol
+                         : which == 0 ? r + size_t(row) * ldr + col
+                         : which == 1 ? k + size_t(row) * ldk + col
+                         : which == 2 ? w + size_t(row) * D + col
+                         : which == 3 ? au + size_t(row) * D + col
+                                      : u + size_t(row) * D + col;
+      const float val = *src;
+      pf[q] = ok ? val : 0.f;
     }
   };
   auto stage = [&]() {

@@ -156,9 +156,9 @@ int kvcm_head_norm_gate(const float* o, int ldo, const float* g, int ldg, const 
                         int ldout, int T, int heads, int d, float eps, hipStream_t s);
 // (short_conv.hip) a short causal convolution per channel over packed runs, its last inputs kept per sequence
 int kvcm_short_conv(const float* in, int ld_in, const float* bias_in, const float* w, const float* bias_out,
-                    const float* state, void* out, int out_dtype, int ld_out, const int* row_seq, const int* positions,
+                    float* state, void* out, int out_dtype, int ld_out, const int* row_seq, const int* positions,
                     const int* ctx_lens, const int* run_start, const int* seq_start, const int* state_slots, int T, int C,
-                    int taps, int act, hipStream_t s);
+                    int taps, int act, int update_state, hipStream_t s);
 int kvcm_short_conv_state(const float* in, int ld_in, const float* bias_in, float* state, const int* run_start,
                           const int* seq_start, const int* seq_end, const int* state_slots, int S, int C, int taps,
                           hipStream_t s);
@@ -184,7 +184,8 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
 int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
                         const float* bc, int ldbc, int off_b, int off_c, const float* a_log, const float* dskip,
                         const float* z, int ldz, void* out, int ldo, float* state, const int* run_start,
-                        const int* seq_start, const int* state_slots, int S, int C, int N, hipStream_t s);
+                        const int* seq_start, const int* state_slots, int S, int C, int N, int prepared, hipStream_t s);
+int kvcm_scan_prepare(float* dt, int lddt, const float* dt_bias, float* z, int ldz, int T, int C, hipStream_t s);
 int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, const float* a_bias, const float* low, int ldlow,
                        const float* w2, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,
                        int d, hipStream_t s);

@@ -28,7 +28,7 @@ __global__ void __launch_bounds__(kWave)
                           const float* __restrict__ a_log, const float* __restrict__ dskip, const float* __restrict__ z,
                           int ldz, T* __restrict__ out, int ldo, float* __restrict__ state,
                           const int* __restrict__ run_start, const int* __restrict__ seq_start,
-                          const int* __restrict__ state_slots, int C, int N) {
+                          const int* __restrict__ state_slots, int C, int N, int prepared) {
   constexpr int U = kScanAhead;
   const int s = blockIdx.y;
   const int sub = threadIdx.x % LPC;
@@ -79,7 +79,7 @@ __global__ void __launch_bounds__(kWave)
       const int r = first + u;
       if (r < r1) {
         const float v = dtv[from][u] + db;
-        const float dt = v > 20.f ? v : log1pf(expf(v));
+        const float dt = prepared ? dtv[from][u] : (v > 20.f ? v : log1pf(expf(v)));
         const float dx = dt * xv[from][u];
         float y = 0.f;
 #pragma unroll
@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(kWave)
         if (owns && sub == 0) {
           y = fmaf(dk, xv[from][u], y);
           const float zz = zv[from][u];
-          store_f(out + size_t(r) * ldo + c, y * (zz / (1.0f + expf(-zz))));
+          store_f(out + size_t(r) * ldo + c, y * (prepared ? zz : zz / (1.0f + expf(-zz))));
         }
       }
     }
@@ -113,15 +113,27 @@ __global__ void __launch_bounds__(kWave)
   }
 }
 
+// For long runs: the step sizes and the gates of all rows at once, in place (dt <- softplus(dt + bias), z <- silu(z)),
+// so that the walk along a run, whose lanes would each repeat them, finds them made.
+__global__ void __launch_bounds__(256)
+    scan_prepare_kernel(float* __restrict__ dt, int lddt, const float* __restrict__ dt_bias, float* __restrict__ z, int ldz, int C) {
+  const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const float v = dt[size_t(r) * lddt + c] + (dt_bias ? dt_bias[c] : 0.f);
+  dt[size_t(r) * lddt + c] = v > 20.f ? v : log1pf(expf(v));
+  const float zz = z[size_t(r) * ldz + c];
+  z[size_t(r) * ldz + c] = zz / (1.0f + expf(-zz));
+}
+
 template <class T>
 int launch_scan(const void* x, int ldx, const float* dt_lin, int lddt, const float* dt_bias, const float* bc, int ldbc,
                 int off_b, int off_c, const float* a_log, const float* dskip, const float* z, int ldz, void* out, int ldo,
                 float* state, const int* run_start, const int* seq_start, const int* state_slots, int S, int C, int N,
-                hipStream_t s) {
+                int prepared, hipStream_t s) {
 #define KVCM_SCAN(LPC, NPL)                                                                                             \
   selective_scan_kernel<T, LPC, NPL><<<dim3((C + kWave / LPC - 1) / (kWave / LPC), S), kWave, 0, s>>>(                   \
       static_cast<const T*>(x), ldx, dt_lin, lddt, dt_bias, bc, ldbc, off_b, off_c, a_log, dskip, z, ldz,               \
-      static_cast<T*>(out), ldo, state, run_start, seq_start, state_slots, C, N)
+      static_cast<T*>(out), ldo, state, run_start, seq_start, state_slots, C, N, prepared)
   if (N <= 1) KVCM_SCAN(1, 1);
   else if (N <= 2) KVCM_SCAN(2, 1);
   else if (N <= 4) KVCM_SCAN(4, 1);
@@ -140,10 +152,12 @@ using namespace kvcm;
 
 // x [T, C] (after its convolution and activation) and out [T, C] in the storage type; dt_lin [T, C], bc [T, ldbc]
 // (B at off_b, C at off_c, N each), z [T, ldz], a_log [C, N], dt_bias, dskip [C], state [slots, C, N]: 32-bit.
+// prepared: dt_lin holds the step sizes and z the gates already (kvcm_scan_prepare).
 extern "C" int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
                                    const float* bc, int ldbc, int off_b, int off_c, const float* a_log, const float* dskip,
                                    const float* z, int ldz, void* out, int ldo, float* state, const int* run_start,
-                                   const int* seq_start, const int* state_slots, int S, int C, int N, hipStream_t s) {
+                                   const int* seq_start, const int* state_slots, int S, int C, int N, int prepared,
+                                   hipStream_t s) {
   if (S == 0) return 0;
   KVCM_REQUIRE(S > 0 && C > 0 && N > 0, "selective_scan: bad sizes S=%d C=%d N=%d", S, C, N);
   KVCM_REQUIRE(N <= 128, "selective_scan: a state of %d per channel is not supported (up to 128)", N);
@@ -152,9 +166,18 @@ extern "C" int kvcm_selective_scan(const void* x, int dtype, int ldx, const floa
                    ldbc >= off_c + N, "selective_scan: row strides too small");
   if (dtype == kF32)
     return launch_scan<float>(x, ldx, dt_lin, lddt, dt_bias, bc, ldbc, off_b, off_c, a_log, dskip, z, ldz, out, ldo, state,
-                              run_start, seq_start, state_slots, S, C, N, s);
+                              run_start, seq_start, state_slots, S, C, N, prepared, s);
   if (dtype == kBF16)
     return launch_scan<bf16_t>(x, ldx, dt_lin, lddt, dt_bias, bc, ldbc, off_b, off_c, a_log, dskip, z, ldz, out, ldo, state,
-                               run_start, seq_start, state_slots, S, C, N, s);
+                               run_start, seq_start, state_slots, S, C, N, prepared, s);
   KVCM_REQUIRE(false, "selective_scan: unknown dtype %d", dtype);
+}
+
+// dt [T, C] <- softplus(dt + dt_bias), z [T, C] <- silu(z), in place; kvcm_selective_scan then runs with prepared = 1.
+extern "C" int kvcm_scan_prepare(float* dt, int lddt, const float* dt_bias, float* z, int ldz, int T, int C, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && C > 0 && lddt >= C && ldz >= C, "scan_prepare: bad sizes T=%d C=%d", T, C);
+  KVCM_REQUIRE(T <= 65535, "scan_prepare: too many rows for one launch (%d)", T);
+  scan_prepare_kernel<<<dim3((C + 255) / 256, T), 256, 0, s>>>(dt, lddt, dt_bias, z, ldz, C);
+  return launch_status("scan_prepare");
 }

@@ -20,10 +20,10 @@ constexpr int kConvMaxTaps = 8;
 template <class TO>
 __global__ void __launch_bounds__(256)
     short_conv_kernel(const float* __restrict__ in, int ld_in, const float* __restrict__ bias_in,
-                      const float* __restrict__ w, const float* __restrict__ bias_out, const float* __restrict__ state,
+                      const float* __restrict__ w, const float* __restrict__ bias_out, float* __restrict__ state,
                       TO* __restrict__ out, int ld_out, const int* __restrict__ row_seq, const int* __restrict__ positions,
                       const int* __restrict__ ctx_lens, const int* __restrict__ run_start, const int* __restrict__ seq_start,
-                      const int* __restrict__ state_slots, int C, int taps, int act) {
+                      const int* __restrict__ state_slots, int C, int taps, int act, int update_state) {
   const int row = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
@@ -35,14 +35,27 @@ __global__ void __launch_bounds__(256)
   const int s = row_seq[row], p = positions[row];
   const int p0 = seq_start[s], r0 = run_start[s], slot = state_slots[s];
   const float bi = bias_in ? bias_in[c] : 0.f;
-  const float* st = slot >= 0 ? state + (size_t(slot) * (taps - 1)) * C + c : nullptr;
+  float* st = slot >= 0 ? state + (size_t(slot) * (taps - 1)) * C + c : nullptr;
   float y = 0.f;
-  for (int j = 0; j < taps; ++j) {
-    const int t = p - (taps - 1) + j;
-    float u = 0.f;
-    if (t >= p0) u = in[size_t(r0 + (t - p0)) * ld_in + c] + bi;
-    else if (t >= 0 && st) u = st[size_t(t - (p0 - (taps - 1))) * C];
-    y = fmaf(w[size_t(c) * taps + j], u, y);
+  float seen[kConvMaxTaps];
+#pragma unroll
+  for (int j = 0; j < kConvMaxTaps; ++j) {
+    seen[j] = 0.f;
+    if (j < taps) {
+      const int t = p - (taps - 1) + j;
+      float u = 0.f;
+      if (t >= p0) u = in[size_t(r0 + (t - p0)) * ld_in + c] + bi;
+      else if (t >= 0 && st) u = st[size_t(t - (p0 - (taps - 1))) * C];
+      seen[j] = u;
+      y = fmaf(w[size_t(c) * taps + j], u, y);
+    }
+  }
+  // a step in which every sequence runs one row: nobody else reads this sequence's state, so the row that read it
+  // leaves the new one (its inputs but the oldest) and the second launch is not needed
+  if (update_state && st) {
+#pragma unroll
+    for (int j = 1; j < kConvMaxTaps; ++j)
+      if (j < taps) st[size_t(j - 1) * C] = seen[j];
   }
   if (bias_out) y += bias_out[c];
   if (act == 1) y = y / (1.0f + expf(-y));
@@ -85,10 +98,11 @@ using namespace kvcm;
 extern "C" {
 
 // in [T, >= C] 32-bit; w [C, taps]; state [slots, taps-1, C] 32-bit; out [T, >= C]; act 0: none, 1: silu.
+// update_state: only for steps in which every sequence runs exactly one row; the state is then written here.
 int kvcm_short_conv(const float* in, int ld_in, const float* bias_in, const float* w, const float* bias_out,
-                    const float* state, void* out, int out_dtype, int ld_out, const int* row_seq, const int* positions,
+                    float* state, void* out, int out_dtype, int ld_out, const int* row_seq, const int* positions,
                     const int* ctx_lens, const int* run_start, const int* seq_start, const int* state_slots, int T, int C,
-                    int taps, int act, hipStream_t s) {
+                    int taps, int act, int update_state, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && C > 0, "short_conv: bad sizes T=%d C=%d", T, C);
   KVCM_REQUIRE(taps >= 1 && taps <= kConvMaxTaps, "short_conv: %d taps are not supported (1 to %d are)", taps, kConvMaxTaps);
@@ -98,10 +112,10 @@ int kvcm_short_conv(const float* in, int ld_in, const float* bias_in, const floa
   const dim3 grid((C + 255) / 256, T);
   if (out_dtype == kF32)
     short_conv_kernel<float><<<grid, 256, 0, s>>>(in, ld_in, bias_in, w, bias_out, state, static_cast<float*>(out), ld_out,
-                                                   row_seq, positions, ctx_lens, run_start, seq_start, state_slots, C, taps, act);
+                                                   row_seq, positions, ctx_lens, run_start, seq_start, state_slots, C, taps, act, update_state);
   else if (out_dtype == kBF16)
     short_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(in, ld_in, bias_in, w, bias_out, state, static_cast<bf16_t*>(out), ld_out,
-                                                    row_seq, positions, ctx_lens, run_start, seq_start, state_slots, C, taps, act);
+                                                    row_seq, positions, ctx_lens, run_start, seq_start, state_slots, C, taps, act, update_state);
   else KVCM_REQUIRE(false, "short_conv: unknown output dtype %d", out_dtype);
   return launch_status("short_conv");
 }

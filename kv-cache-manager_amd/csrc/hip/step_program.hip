@@ -103,6 +103,7 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_attention_window_pool),
     KVCM_ENTRY(kvcm_attention_window_pool_tiles),
     KVCM_ENTRY(kvcm_selective_scan),
+    KVCM_ENTRY(kvcm_scan_prepare),
     KVCM_ENTRY(kvcm_delta_prepare),
     KVCM_ENTRY(kvcm_delta_scan),
 };

@@ -90,7 +90,7 @@ def _declare(lib):
     fn("kvcm_widen", vp, vp, C.c_longlong, vp)
     fn("kvcm_rmsnorm_chain", vp, vp, vp, vp, vp, f, vp, vp, vp, vp, i, i, i, f, vp)
     fn("kvcm_head_norm_gate", vp, i, vp, i, vp, vp, i, i, i, i, i, f, vp)
-    fn("kvcm_short_conv", vp, i, vp, vp, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_short_conv", vp, i, vp, vp, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_short_conv_state", vp, i, vp, vp, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_rotary_pairs_table", vp, vp, i, i, f, vp)
     fn("kvcm_rotate_store", vp, i, vp, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
@@ -98,7 +98,8 @@ def _declare(lib):
     fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp)
     fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
     fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, vp)
-    fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
+    fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_scan_prepare", vp, i, vp, vp, i, i, i, vp)
     fn("kvcm_delta_prepare", vp, i, vp, i, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_delta_scan", vp, i, vp, i, vp, i, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, vp)
     lib.kvcm_gemm_library_workspace_bytes.restype = C.c_longlong
@@ -1012,10 +1013,11 @@ def head_norm_gate(o, gate, weight, out, heads, d, eps):
     return out
 
 
-def short_conv(x, weight, out, step, state, bias_in=None, bias_out=None, activation=None, rows=None):
+def short_conv(x, weight, out, step, state, bias_in=None, bias_out=None, activation=None, rows=None, update_state=False):
     """Causal convolution per channel over the step's packed runs.  x: 32-bit rows [T, >= C]; weight [C, taps];
     state [slots, taps-1, C] (the sequences' last inputs, read here); out [T, >= C].  ``step`` brings row_seq,
-    positions, ctx_lens, run_start, seq_start, state_slots."""
+    positions, ctx_lens, run_start, seq_start, state_slots.  ``update_state``: for steps in which every sequence runs one
+    row only; the rows then leave the new state themselves and ``short_conv_state`` is not called."""
     C, taps = weight.shape
     T = out.shape[0] if rows is None else rows
     _f32rows(x, "x", C)
@@ -1032,7 +1034,8 @@ def short_conv(x, weight, out, step, state, bias_in=None, bias_out=None, activat
         _i32(getattr(step, name), name, T)
     _call("kvcm_short_conv", _ptr(x), x.stride(0), _ptr(bias_in), _ptr(weight), _ptr(bias_out), _ptr(state), _ptr(out),
           _DT[out.dtype], out.stride(0), _ptr(step.row_seq), _ptr(step.positions), _ptr(step.ctx_lens), _ptr(step.run_start),
-          _ptr(step.seq_start), _ptr(step.state_slots), T, C, taps, 1 if activation == "silu" else 0, _stream())
+          _ptr(step.seq_start), _ptr(step.state_slots), T, C, taps, 1 if activation == "silu" else 0,
+          1 if (update_state and taps > 1) else 0, _stream())
     return out
 
 
@@ -1155,9 +1158,10 @@ def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_st
           d, dv, B, float(scale), int(window), int(P), E, _stream())
 
 
-def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, state, step):
+def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, state, step, prepare=False):
     """The selective scan of the step's runs (csrc/hip/selective_scan.hip).  x, out [T, C] in the compute dtype;
-    dt_lin [T, C], bc rows with B at off_b and C at off_c, z rows: 32-bit; state [slots, C, N]."""
+    dt_lin [T, C], bc rows with B at off_b and C at off_c, z rows: 32-bit; state [slots, C, N].  ``prepare``: the step
+    sizes and gates of all rows are made first, in place in dt_lin and z, by a launch of their own (pays for long runs)."""
     C, N = a_log.shape
     _rows2d(x, "x")
     _rows2d(out, "out")
@@ -1170,9 +1174,11 @@ def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, s
     _f32(dskip, "dskip", C)
     _need(state.dtype == torch.float32 and state.is_contiguous() and state.is_cuda and tuple(state.shape[1:]) == (C, N),
           "state must be float32 [slots, C, N]")
+    if prepare:
+        _call("kvcm_scan_prepare", _ptr(dt_lin), dt_lin.stride(0), _ptr(dt_bias), _ptr(z), z.stride(0), out.shape[0], C, _stream())
     _call("kvcm_selective_scan", _ptr(x), _DT[x.dtype], x.stride(0), _ptr(dt_lin), dt_lin.stride(0), _ptr(dt_bias), _ptr(bc),
           bc.stride(0), off_b, off_c, _ptr(a_log), _ptr(dskip), _ptr(z), z.stride(0), _ptr(out), out.stride(0), _ptr(state),
-          _ptr(step.run_start), _ptr(step.seq_start), _ptr(step.state_slots), step.seqs, C, N, _stream())
+          _ptr(step.run_start), _ptr(step.seq_start), _ptr(step.state_slots), step.seqs, C, N, 1 if prepare else 0, _stream())
     return out
 
 

@@ -96,8 +96,10 @@ class ConvWindowPoolAttention(Mixer):
         proj = linear32(self.ctx, step, h, w["w_qkv"], "cwp_proj")
         mixed = step.ws("cwp_conv", (T, self.channels), torch.float32)
         conv_state = self.caches["conv"][0].slots(self.caches["conv"][1]) if K > 1 else None
-        ops.short_conv(proj, w["conv"], mixed, step, conv_state, bias_in=w["bias"])
-        ops.short_conv_state(proj, conv_state, step, K, bias_in=w["bias"])
+        single = step.max_run == 1      # every sequence runs one row: the convolution leaves the new state itself
+        ops.short_conv(proj, w["conv"], mixed, step, conv_state, bias_in=w["bias"], update_state=single)
+        if not single:
+            ops.short_conv_state(proj, conv_state, step, K, bias_in=w["bias"])
         q = step.ws("cwp_q", (T, self.nh * self.d))
         slots = step.slots(g) if self.cache_owner else None
         ops.rotate_store(mixed, q, self.nh, self.nkv, self.d, self.dv, cos_sin=self.position.pairs_table(step),

@@ -62,14 +62,17 @@ class SelectiveScanMixer(_StatefulMixer):
         xz = linear32(self.ctx, step, h, w["w_in"], "scan_xz")
         conv_state = self.state("conv") if K > 1 else None
         x = step.ws("scan_x", (step.rows, C))
-        ops.short_conv(xz, w["conv"], x, step, conv_state, bias_out=w["conv_bias"], activation="silu")
-        ops.short_conv_state(xz, conv_state, step, K)
+        single = step.max_run == 1      # every sequence runs one row: the convolution leaves the new state itself
+        ops.short_conv(xz, w["conv"], x, step, conv_state, bias_out=w["conv_bias"], activation="silu", update_state=single)
+        if not single:
+            ops.short_conv_state(xz, conv_state, step, K)
         # the step size's low-rank input feeds a product (compute dtype); B and C enter the recurrence (32-bit)
         low = _linear(self.ctx, step, x, w["w_x"][:R], "scan_dt_low")
         bc = _linear(self.ctx, step, x, w["w_x"][R:], "scan_bc", dtype=torch.float32)
         dt = _linear(self.ctx, step, low, w["w_dt"], "scan_dt", dtype=torch.float32)
         y = step.ws("scan_y", (step.rows, C))
-        ops.selective_scan(x, dt, w["dt_bias"], bc, 0, N, w["a_log"], w["d_skip"], xz[:, C:], y, self.state("scan"), step)
+        ops.selective_scan(x, dt, w["dt_bias"], bc, 0, N, w["a_log"], w["d_skip"], xz[:, C:], y, self.state("scan"), step,
+                           prepare=step.max_run >= 16)
         return linear32(self.ctx, step, y, w["w_o"], "scan_out")
 
 
@@ -113,9 +116,16 @@ class GeneralDeltaMixer(_StatefulMixer):
         ops, p, w = self.ctx.ops, self.params, self.w
         heads, d = p["heads"], p["dim"]
         D, T = heads * d, step.rows
-        proj = _linear(self.ctx, step, h, w["w_proj"], "delta_proj", dtype=torch.float32)
-        r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
-        low = proj[:, 5 * D:]
+        if h.dtype == torch.bfloat16 and ops.library_takes(T, 4 * D, h.shape[1]):
+            # many rows: r, k, v, g through the vendor library; what enters the recurrence's decay and removal rate keeps its sums
+            rkvg = linear32(self.ctx, step, h, w["w_proj"][:4 * D], "delta_rkvg")
+            rest = _linear(self.ctx, step, h, w["w_proj"][4 * D:], "delta_a_low", dtype=torch.float32)
+            r, k, v, g = (rkvg[:, i * D:(i + 1) * D] for i in range(4))
+            a, low = rest[:, :D], rest[:, D:]
+        else:
+            proj = _linear(self.ctx, step, h, w["w_proj"], "delta_proj", dtype=torch.float32)
+            r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
+            low = proj[:, 5 * D:]
         decay, au, u = (step.ws(n, (T, D), torch.float32) for n in ("delta_w", "delta_au", "delta_u"))
         ops.delta_prepare(k, a, w["a_bias"], low, w["w2"], w["w0"], decay, au, u, heads, d, T)
         o = step.ws("delta_o", (T, D), torch.float32)

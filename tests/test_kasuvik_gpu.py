@@ -120,6 +120,36 @@ def test_short_convolution_over_cut_runs_with_state(taps):
         np.testing.assert_allclose(got_act[s], want_act[s], atol=1e-5)
 
 
+@pytest.mark.parametrize("taps", [2, 4])
+def test_short_convolution_single_rows_leave_their_own_state(taps):
+    """Steps in which every sequence runs one row: the convolution kernel writes the state itself; a prompt portion
+    before and after goes through the second launch, and both must hand over to one another."""
+    from kvcm_amd import ops
+    rng = np.random.default_rng(10 + taps)
+    C, lengths = 21, (17, 9)
+    u = [rng.normal(size=(n, C)) for n in lengths]
+    w = rng.normal(size=(C, taps))
+    want = [plain.short_conv(x, w) for x in u]
+    state = torch.full((2, taps - 1, C), 9.0, device=DEV)
+    got = [np.zeros_like(x) for x in u]
+    plan = [[(0, 0, 3), (1, 0, 1)]] + [[(0, 3 + i, 1), (1, 1 + i, 1)] for i in range(5)] + [[(0, 8, 4)], [(1, 6, 1), (0, 12, 1)],
+            [(0, 13, 4), (1, 7, 2)]]
+    for runs in plan:
+        step = Step(runs)
+        single = all(n == 1 for _, _, n in runs)
+        x = dev(np.concatenate([u[s][p:p + n] for s, p, n in runs]))
+        out = torch.empty(step.rows, C, device=DEV)
+        ops.short_conv(x, dev(w), out, step, state, update_state=single)
+        if not single:
+            ops.short_conv_state(x, state, step, taps)
+        r = 0
+        for s, p, n in runs:
+            got[s][p:p + n] = out[r:r + n].cpu().numpy()
+            r += n
+    np.testing.assert_allclose(got[0], want[0], atol=1e-5)
+    np.testing.assert_allclose(got[1], want[1], atol=1e-5)
+
+
 def _pages(rng, tokens, B, nkv, d, dv, P, dtype):
     n = -(-tokens // B)
     order = rng.permutation(n + 3)[:n]                # pages in no order, three left out
