@@ -47,7 +47,7 @@ def make_engine(a, ec: EngineConfig):
     --random-weights with --sizes NAME | --config-json FILE and --weights-seed."""
     import torch
 
-    from ..config.model_config import LlamaConfig
+    from ..config.model_config import architecture_name
     from ..engine.engine import Engine
     from ..weights.random_init import random_tensors
     model_dir = a.str("model", a.str("weights", ""))
@@ -60,7 +60,7 @@ def make_engine(a, ec: EngineConfig):
             if name not in NAMED_SIZES:
                 raise ValueError(f"unknown --sizes {name!r}; known: {sorted(NAMED_SIZES)}")
             raw = NAMED_SIZES[name]
-        arch = raw.get("architectures", ["LlamaForCausalLM"])[0]
+        arch = architecture_name(raw, "LlamaForCausalLM")
         from .. import architectures  # noqa: F401
         from ..registry import ARCHITECTURES
         cfg = ARCHITECTURES.get(arch).config_class.from_dict(raw)

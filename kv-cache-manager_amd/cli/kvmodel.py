@@ -35,9 +35,10 @@ def main(argv=None):
         import torch
 
         from .. import architectures  # noqa: F401
+        from ..config.model_config import architecture_name
         from ..registry import ARCHITECTURES
         from ..weights.random_init import write_model_dir
-        arch = raw.get("architectures", ["LlamaForCausalLM"])[0]
+        arch = architecture_name(raw, "LlamaForCausalLM")
         cfg = ARCHITECTURES.get(arch).config_class.from_dict(raw)
         path = write_model_dir(out, arch, cfg, seed, torch.bfloat16 if dtype in ("bf16", "bfloat16") else torch.float32,
                                std=std, norm_jitter=jitter)

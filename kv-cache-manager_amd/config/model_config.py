@@ -20,18 +20,27 @@ class ConfigError(ValueError):
 MAX_HEAD_DIM = 256
 
 
+def architecture_name(raw: dict, default=None):
+    """The model class a configuration names: ``architectures[0]`` or, where a folder names one class as a string,
+    ``architecture``."""
+    archs = raw.get("architectures")
+    if isinstance(archs, list) and archs and isinstance(archs[0], str):
+        return archs[0]
+    if isinstance(raw.get("architecture"), str):
+        return raw["architecture"]
+    return default
+
+
 def read_config_json(model_dir):
     path = os.path.join(model_dir, "config.json")
     if not os.path.isfile(path):
         raise ConfigError(f"{model_dir}: no config.json")
     with open(path) as f:
         raw = json.load(f)
-    archs = raw.get("architectures")
-    if archs is None and isinstance(raw.get("architecture"), str):      # some model folders name one class, as a string
-        archs = [raw["architecture"]]
-    if not archs or not isinstance(archs, list) or not isinstance(archs[0], str):
+    name = architecture_name(raw)
+    if name is None:
         raise ConfigError(f"{path}: 'architectures' (or 'architecture') must name the model class, e.g. [\"LlamaForCausalLM\"]")
-    return archs[0], raw
+    return name, raw
 
 
 @dataclass(frozen=True)

@@ -120,12 +120,24 @@ __device__ __forceinline__ void unpack_piece(const bf16_t* p, float* f) {
   f[6] = bf16_bits_to_float(v.w & 0xffffu); f[7] = bf16_bits_to_float(v.w >> 16);
 }
 
+// (four pieces of the row are requested before the first is multiplied: a load per trip of the loop would wait for
+// each one in turn)
 template <class T>
 __device__ __forceinline__ float dot_row(const float* qs, const T* kp, int d, bool wide) {
   constexpr int N = RowPiece<T>::N;
   float s = 0.f;
   if (wide) {
-    for (int i = 0; i < d; i += N) {
+    int i = 0;
+    for (; i + 4 * N <= d; i += 4 * N) {
+      float f[4][N];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) unpack_piece(kp + i + g * N, f[g]);
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int e = 0; e < N; ++e) s = fmaf(qs[i + g * N + e], f[g][e], s);
+    }
+    for (; i < d; i += N) {
       float f[N];
       unpack_piece(kp + i, f);
 #pragma unroll
@@ -230,20 +242,29 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
       const int j_lo = first > c0 ? first - c0 : 0;
       const int j_hi = ctx - c0 < kWave ? ctx - c0 : kWave;
       if (wide_v) {
-        for (int j0 = (j_lo / N) * N; j0 < j_hi; j0 += N) {      // N tokens of one page at a time
-          const int tj = c0 + j0;
-          const T* vp = vcache + size_t(table[tj / B]) * vpage + kvh * vhead + tj % B;      // [column][slot]
+        // all of the chunk's pieces (N tokens of one page each) are requested at once, from places clamped into the
+        // context; probabilities of tokens before the window are zero, values beyond the context are cut
+        const int last_piece = ((ctx - 1) / N) * N;
 #pragma unroll
-          for (int i = 0; i < COLS; ++i) {
-            const int cc = lane + i * kWave;
-            if (cc < dv) {
-              float f[N];
-              unpack_piece(vp + size_t(cc) * B, f);
+        for (int i = 0; i < COLS; ++i) {
+          if (i * kWave >= dv) break;      // the same for every lane: 64 columns at a time, each with its own trip of loads
+          const int cc = lane + i * kWave;
+          const int col = cc < dv ? cc : dv - 1;
+          float f[kWave / N][N];
 #pragma unroll
-              for (int e = 0; e < N; ++e)
-                if (j0 + e >= j_lo && j0 + e < j_hi) o[i] = fmaf(ps[j0 + e], f[e], o[i]);      // beyond the context: stale values, never used
-            }
+          for (int g = 0; g < kWave / N; ++g) {
+            const int tj = c0 + g * N < last_piece ? c0 + g * N : last_piece;
+            unpack_piece(vcache + size_t(table[tj / B]) * vpage + kvh * vhead + size_t(col) * B + tj % B, f[g]);
           }
+          float acc = o[i];
+#pragma unroll
+          for (int g = 0; g < kWave / N; ++g)
+#pragma unroll
+            for (int e = 0; e < N; ++e) {
+              const int j = g * N + e;
+              acc = fmaf(ps[j], j < j_hi ? f[g][e] : 0.f, acc);
+            }
+          if (cc < dv) o[i] = acc;
         }
       } else {
         for (int j = j_lo; j < j_hi; ++j) {

@@ -83,9 +83,47 @@ __global__ void __launch_bounds__(256)
   const int first_token_chunk = t_lo / kChunk, last_token_chunk = p_last / kChunk;
   const int chunks = block_chunks + (last_token_chunk - first_token_chunk + 1);
 
+  // A chunk of tokens on its way from the pages to LDS, held in registers meanwhile: the next chunk is requested
+  // before the current one is multiplied.  Loads are unconditional, from places clamped into the sequence, and
+  // masked afterwards (a branch around a load would make each wait for the one before).
+  constexpr int KQ = (kChunk * (DP / 8) + 255) / 256, VQ = (DVP * (kChunk / 8) + 255) / 256;
+  uint4 kreg[KQ], vreg[VQ];
+  auto request_tokens = [&](int c0) {
+#pragma unroll
+    for (int qq = 0; qq < KQ; ++qq) {
+      const int e = tid + qq * 256;
+      const int key = (e / (DP / 8)) % kChunk, k = (e % (DP / 8)) * 8, t = c0 + key;
+      const int tc = t <= p_last ? t : p_last, kc = k < d ? k : d - 8;
+      const uint4 v = *reinterpret_cast<const uint4*>(kcache + ((size_t(table[tc / B]) * nkv + kvh) * B + tc % B) * d + kc);
+      kreg[qq] = (t <= p_last && k < d) ? v : uint4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int qq = 0; qq < VQ; ++qq) {
+      const int e = tid + qq * 256;
+      const int cc = (e / (kChunk / 8)) % DVP, piece = e % (kChunk / 8), t = c0 + piece * 8;
+      const int tc = t <= p_last ? t : (p_last / 8) * 8, ccl = cc < dv ? cc : dv - 1;
+      uint4 v = *reinterpret_cast<const uint4*>(vcache + ((size_t(table[tc / B]) * nkv + kvh) * dv + ccl) * B + tc % B);
+      v = keep_first_bf16(v, p_last + 1 - t < 8 ? p_last + 1 - t : 8);      // beyond the newest token: whatever was there
+      vreg[qq] = cc < dv ? v : uint4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto stage_tokens = [&]() {
+#pragma unroll
+    for (int qq = 0; qq < KQ; ++qq) {
+      const int e = tid + qq * 256;
+      if (e < kChunk * (DP / 8)) *reinterpret_cast<uint4*>(&Ks[e / (DP / 8)][(e % (DP / 8)) * 8]) = kreg[qq];
+    }
+#pragma unroll
+    for (int qq = 0; qq < VQ; ++qq) {
+      const int e = tid + qq * 256;
+      if (e < DVP * (kChunk / 8)) *reinterpret_cast<uint4*>(&Vt[e / (kChunk / 8)][(e % (kChunk / 8)) * 8]) = vreg[qq];
+    }
+  };
+
   for (int c = 0; c < chunks; ++c) {
     const bool pooled = c < block_chunks;
     const int c0 = pooled ? c * kChunk : (first_token_chunk + (c - block_chunks)) * kChunk;
+    if (!pooled && c == block_chunks) request_tokens(c0);      // the first chunk of tokens: nobody asked for it yet
     __syncthreads();      // the chunk before is done with Ks, Vt and Ps
     if (pooled) {
       for (int e = tid; e < kChunk * (DP / 8); e += 256) {
@@ -109,24 +147,10 @@ __global__ void __launch_bounds__(256)
         Vt[cc][key] = float_to_bf16_bits(x);
       }
     } else {
-      for (int e = tid; e < kChunk * (DP / 8); e += 256) {
-        const int key = e / (DP / 8), k = (e % (DP / 8)) * 8, t = c0 + key;
-        uint4 v = {0u, 0u, 0u, 0u};
-        if (t <= p_last && k < d)
-          v = *reinterpret_cast<const uint4*>(kcache + ((size_t(table[t / B]) * nkv + kvh) * B + t % B) * d + k);
-        *reinterpret_cast<uint4*>(&Ks[key][k]) = v;
-      }
-      for (int e = tid; e < DVP * (kChunk / 8); e += 256) {
-        const int cc = e / (kChunk / 8), piece = e % (kChunk / 8), t = c0 + piece * 8;
-        uint4 v = {0u, 0u, 0u, 0u};
-        if (t <= p_last && cc < dv) {
-          v = *reinterpret_cast<const uint4*>(vcache + ((size_t(table[t / B]) * nkv + kvh) * dv + cc) * B + t % B);
-          v = keep_first_bf16(v, p_last + 1 - t < 8 ? p_last + 1 - t : 8);      // beyond the newest token: whatever was there
-        }
-        *reinterpret_cast<uint4*>(&Vt[cc][piece * 8]) = v;
-      }
+      stage_tokens();
     }
     __syncthreads();
+    if (!pooled && c + 1 < chunks) request_tokens(c0 + kChunk);      // on its way while this chunk is multiplied
 
     // scores of 16 rows x 64 keys: four column tiles
     f32x4 sc[4];

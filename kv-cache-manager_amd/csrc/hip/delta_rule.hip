@@ -23,12 +23,13 @@ namespace kvcm {
 constexpr int kDeltaTile = 8;      // tokens staged at once
 
 // one wave per (row, head).  The decay's logit is a two-step projection whose second step runs here in 32-bit:
-// w_lin[c] = sum_j w2[c, j] * tanh(low[j]), low = the first step's output (rank values a row).
+// w_lin[c] = sum_j w2[c, j] * tanh(low[j]), low = the first step's output (rank values a row); w2 comes transposed,
+// [rank, heads*d].
 constexpr int kDeltaMaxRank = 256;
 __global__ void __launch_bounds__(256)
     delta_prepare_kernel(const float* __restrict__ k, int ldk, const float* __restrict__ a_lin, int lda,
                          const float* __restrict__ a_bias, const float* __restrict__ low, int ldlow,
-                         const float* __restrict__ w2, int rank, const float* __restrict__ w0,
+                         const float* __restrict__ w2t, int rank, const float* __restrict__ w0,
                          float* __restrict__ w_out, float* __restrict__ au_out, float* __restrict__ u_out, long long items,
                          int heads, int d) {
   __shared__ float th[256 / kWave][kDeltaMaxRank];
@@ -51,8 +52,7 @@ __global__ void __launch_bounds__(256)
     const float u = kr[i] * inv;
     const float a = 1.0f / (1.0f + expf(-(a_lin[size_t(row) * lda + col + i] + a_bias[col + i])));
     float wl = 0.f;
-    const float* w2r = w2 + (col + i) * rank;
-    for (int j = 0; j < rank; ++j) wl = fmaf(w2r[j], th[wave][j], wl);
+    for (int j = 0; j < rank; ++j) wl = fmaf(w2t[size_t(j) * D + col + i], th[wave][j], wl);      // neighbours read neighbours
     const float g = 1.0f / (1.0f + expf(-(wl + w0[col + i])));
     w_out[size_t(row) * D + col + i] = expf(-rate * g);
     au_out[size_t(row) * D + col + i] = a * u;
@@ -173,9 +173,9 @@ using namespace kvcm;
 extern "C" {
 
 // k, a_lin: 32-bit rows with heads*d columns each (at their own strides); low: 32-bit rows of `rank` columns;
-// w2 [heads*d, rank], a_bias, w0 [heads*d]; w_out, au_out, u_out [T, heads*d]: all 32-bit.
+// w2t [rank, heads*d] (the second step's matrix, transposed), a_bias, w0 [heads*d]; w_out, au_out, u_out [T, heads*d]: all 32-bit.
 int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, const float* a_bias, const float* low, int ldlow,
-                       const float* w2, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,
+                       const float* w2t, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,
                        int d, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && heads > 0 && d > 0, "delta_prepare: bad sizes T=%d heads=%d d=%d", T, heads, d);
@@ -184,7 +184,7 @@ int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, con
   const long long items = static_cast<long long>(T) * heads;
   const long long blocks = (items + 3) / 4;
   KVCM_REQUIRE(blocks < (1ll << 31), "delta_prepare: too many rows");
-  delta_prepare_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(k, ldk, a_lin, lda, a_bias, low, ldlow, w2, rank, w0, w_out,
+  delta_prepare_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(k, ldk, a_lin, lda, a_bias, low, ldlow, w2t, rank, w0, w_out,
                                                                      au_out, u_out, items, heads, d);
   return launch_status("delta_prepare");
 }

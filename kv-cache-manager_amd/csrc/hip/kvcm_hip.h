@@ -187,7 +187,7 @@ int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, 
                         const int* seq_start, const int* state_slots, int S, int C, int N, int prepared, hipStream_t s);
 int kvcm_scan_prepare(float* dt, int lddt, const float* dt_bias, float* z, int ldz, int T, int C, hipStream_t s);
 int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, const float* a_bias, const float* low, int ldlow,
-                       const float* w2, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,
+                       const float* w2t, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,
                        int d, hipStream_t s);
 int kvcm_delta_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* w, const float* au,
                     const float* u, float* o, int ldo, float* state, const int* run_start, const int* seq_start,

@@ -1182,22 +1182,22 @@ def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, s
     return out
 
 
-def delta_prepare(k, a_lin, a_bias, low, w2, w0, w_out, au_out, u_out, heads, d, rows):
+def delta_prepare(k, a_lin, a_bias, low, w2t, w0, w_out, au_out, u_out, heads, d, rows):
     """(decay, removal rate times unit key, unit key) of every row and head from the projections; ``low`` is the
-    first step of the decay's projection [T, rank], ``w2`` [heads*d, rank] its second step."""
+    first step of the decay's projection [T, rank], ``w2t`` [rank, heads*d] its second step's matrix, transposed."""
     D = heads * d
     for t, n in ((k, "k"), (a_lin, "a_lin")):
         _f32rows(t, n, D)
-    rank = w2.shape[1]
+    rank = w2t.shape[0]
     _f32rows(low, "low", rank)
-    _need(w2.dtype == torch.float32 and w2.is_contiguous() and w2.is_cuda and w2.shape[0] == D, "w2 must be contiguous float32 [heads*d, rank]")
+    _need(w2t.dtype == torch.float32 and w2t.is_contiguous() and w2t.is_cuda and w2t.shape[1] == D, "w2t must be contiguous float32 [rank, heads*d]")
     for t, n in ((a_bias, "a_bias"), (w0, "w0")):
         _f32(t, n, D)
     for t, n in ((w_out, "w_out"), (au_out, "au_out"), (u_out, "u_out")):
         _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and t.shape[0] >= rows and t.shape[1] == D,
               f"{n} must be contiguous float32 [T, heads*d]")
     _call("kvcm_delta_prepare", _ptr(k), k.stride(0), _ptr(a_lin), a_lin.stride(0), _ptr(a_bias), _ptr(low), low.stride(0),
-          _ptr(w2), rank, _ptr(w0), _ptr(w_out), _ptr(au_out), _ptr(u_out), rows, heads, d, _stream())
+          _ptr(w2t), rank, _ptr(w0), _ptr(w_out), _ptr(au_out), _ptr(u_out), rows, heads, d, _stream())
 
 
 def delta_scan(r, k, v, w, au, u, o, state, step, heads, dk, dv):

@@ -20,7 +20,9 @@ def linear32(ctx, step, x, w, name, exact=False):
     """x @ w^T as 32-bit rows for a consumer that computes in 32-bit.  The products of this package write their
     32-bit sums as they are.  A many-row product that the vendor library would take runs there with a bfloat16
     result that is widened afterwards (the library's kernels are several times faster at those shapes), unless
-    ``exact``: what enters a recurrence keeps its 32-bit sums at every row count."""
+    ``exact``: what enters a recurrence keeps its 32-bit sums at every row count.  (Few-row products stay split along K
+    with a second launch that adds the slices up: run unsplit they were slower by more than that launch costs,
+    0.71 -> 0.80 ms a decode step at width 2048, 1.25 -> 1.49 ms at 4096.)"""
     ops = ctx.ops
     M, N, K = x.shape[0], w.shape[0], w.shape[1]
     if not exact and x.dtype == torch.bfloat16 and ops.library_takes(M, N, K):

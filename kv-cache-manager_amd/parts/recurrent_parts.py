@@ -69,7 +69,7 @@ class SelectiveScanMixer(_StatefulMixer):
         # the step size's low-rank input feeds a product (compute dtype); B and C enter the recurrence (32-bit)
         low = _linear(self.ctx, step, x, w["w_x"][:R], "scan_dt_low")
         bc = _linear(self.ctx, step, x, w["w_x"][R:], "scan_bc", dtype=torch.float32)
-        dt = _linear(self.ctx, step, low, w["w_dt"], "scan_dt", dtype=torch.float32)
+        dt = linear32(self.ctx, step, low, w["w_dt"], "scan_dt", exact=True)
         y = step.ws("scan_y", (step.rows, C))
         ops.selective_scan(x, dt, w["dt_bias"], bc, 0, N, w["a_log"], w["d_skip"], xz[:, C:], y, self.state("scan"), step,
                            prepare=step.max_run >= 16)
@@ -100,6 +100,7 @@ class GeneralDeltaMixer(_StatefulMixer):
         super().bind(tensors)
         D = self.params["heads"] * self.params["dim"]
         self.rank = self.w["w2"].shape[1]
+        self.w["w2"] = self.w["w2"].t().contiguous()      # [rank, heads*dim]: the kernel's lanes read neighbours
         if self.w["w_proj"].shape[0] != 5 * D + self.rank:
             raise ValueError(f"general_delta {self.prefix!r}: the two steps of the decay's projection do not agree on their rank "
                              f"({self.w['w_proj'].shape[0] - 5 * D} and {self.rank})")
@@ -123,7 +124,7 @@ class GeneralDeltaMixer(_StatefulMixer):
             r, k, v, g = (rkvg[:, i * D:(i + 1) * D] for i in range(4))
             a, low = rest[:, :D], rest[:, D:]
         else:
-            proj = _linear(self.ctx, step, h, w["w_proj"], "delta_proj", dtype=torch.float32)
+            proj = linear32(self.ctx, step, h, w["w_proj"], "delta_proj", exact=True)
             r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
             low = proj[:, 5 * D:]
         decay, au, u = (step.ws(n, (T, D), torch.float32) for n in ("delta_w", "delta_au", "delta_u"))

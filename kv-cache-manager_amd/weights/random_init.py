@@ -79,6 +79,9 @@ def index_values(key: int, count: int, modulus: int = INDEX_MODULUS) -> np.ndarr
 def random_tensor(seed: int, name: str, shape, role: str, dtype=torch.bfloat16, std=0.02, norm_jitter=0.0, device="cpu"):
     """One tensor of the rule.  role "vector": 1 + norm_jitter * n; "index": int32 in [0, INDEX_MODULUS);
     else std * n.  On a GPU the fill kernel makes the values in place."""
+    if any(n < 0 for n in shape):
+        raise ValueError(f"{name}: a size of this tensor is left to the checkpoint ({tuple(shape)}); random weights need it in "
+                         "the configuration")
     key = tensor_key(seed, name)
     dev = torch.device(device)
     count = int(np.prod(shape)) if len(shape) else 1

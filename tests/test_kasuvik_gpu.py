@@ -275,7 +275,7 @@ def test_delta_rule_against_the_plain_recurrence():
                                        for s, p, n in runs]))
             r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
             w, au, u, o = (torch.empty(T, D, device=DEV) for _ in range(4))
-            ops.delta_prepare(k, a, dev(ab), proj[:, 5 * D:], dev(w2), dev(w0), w, au, u, heads, d, T)
+            ops.delta_prepare(k, a, dev(ab), proj[:, 5 * D:], dev(w2.T.copy()), dev(w0), w, au, u, heads, d, T)
             ops.delta_scan(r, k, v, w, au, u, o, state, step, heads, d, d)
             out = torch.empty(T, D, device=DEV)
             ops.head_norm_gate(o, g, dev(nw), out, heads, d, eps)
