@@ -48,7 +48,9 @@ __global__ void __launch_bounds__(256)
   const int* table = tables + size_t(s) * table_stride;
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
   const int col = lane % 16, quad = lane / 16;
-  const float f = head_scale ? scale * head_scale[head] : scale;
+  // scores are kept in units of log 2 (the factor rides along with the scale), so that the exponentials are the
+  // hardware's exp2: a bfloat16 probability keeps 8 bits of it
+  const float f = (head_scale ? scale * head_scale[head] : scale) * 1.44269504088896341f;
 
   // this wave's 16 query rows as first operands (row = lane % 16, k = 8 * (lane / 16) .. + 8 of every 32)
   bf16x8 qf[KS];
@@ -176,14 +178,13 @@ __global__ void __launch_bounds__(256)
         sc[ct][i] = sv;
         mx = fmaxf(mx, sv);
       }
-#pragma unroll
-      for (int x = 8; x > 0; x >>= 1) mx = fmaxf(mx, __shfl_xor(mx, x, kWave));
+      mx = group_max<16>(mx);
       const float m_new = fmaxf(m[i], mx);
-      alpha[i] = expf(m[i] - m_new);
+      alpha[i] = __builtin_amdgcn_exp2f(m[i] - m_new);
       float add = 0.f;
 #pragma unroll
       for (int ct = 0; ct < 4; ++ct) {
-        const float p = vis[ct] ? expf(sc[ct][i] - m_new) : 0.f;
+        const float p = vis[ct] ? __builtin_amdgcn_exp2f(sc[ct][i] - m_new) : 0.f;
         const uint16_t pb = float_to_bf16_bits(p);
         Ps[wave][quad * 4 + i][ct * 16 + col] = pb;
         add += bf16_bits_to_float(pb);      // the sum of what is multiplied, so that the weights add up to one
@@ -208,9 +209,7 @@ __global__ void __launch_bounds__(256)
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    float l = lsum[i];
-#pragma unroll
-    for (int x = 8; x > 0; x >>= 1) l += __shfl_xor(l, x, kWave);
+    const float l = group_sum<16>(lsum[i]);
     const int row = wave * 16 + quad * 4 + i;
     if (row < nrows) {
       const float inv = 1.0f / l;

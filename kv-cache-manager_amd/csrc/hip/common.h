@@ -91,6 +91,17 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+template <int G>
+__device__ __forceinline__ float group_max(float v) {      // as group_sum, the largest instead of the sum
+  if constexpr (G >= 2) v = fmaxf(v, dpp_take<0xB1>(v));
+  if constexpr (G >= 4) v = fmaxf(v, dpp_take<0x4E>(v));
+  if constexpr (G >= 8) v = fmaxf(v, dpp_take<0x141>(v));
+  if constexpr (G >= 16) v = fmaxf(v, dpp_take<0x140>(v));
+  if constexpr (G >= 32) v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  if constexpr (G >= 64) v = fmaxf(v, __shfl_xor(v, 32, kWave));
+  return v;
+}
+
 // Sum over a block of THREADS threads (a multiple of 64); every thread gets the result.  The
 // order of additions depends on THREADS only.
 template <int THREADS>
