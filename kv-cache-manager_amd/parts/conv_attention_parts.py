@@ -124,7 +124,8 @@ class ParallelMixers(Mixer):
     """Two mixers side by side on the same input; the result is combine * (n(left) * w_left + n(right) * w_right),
     n: division by the root mean square over the model width (eps), the weights plain multipliers.  The two
     outputs are handed on as they are (BranchPair): the norm that adds the result to the stream combines them.
-    params: left, right (PartSpecs of mixers), eps, combine (default 0.5), left_weight, right_weight (checkpoint
+    The epsilon of these two norms is that of the norm which adds the result (one chain, one epsilon).
+    params: left, right (PartSpecs of mixers), combine (default 0.5), left_weight, right_weight (checkpoint
     names after the prefix, defaults "left.out", "right.out")."""
 
     capturable = True
