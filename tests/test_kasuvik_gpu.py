@@ -478,3 +478,28 @@ def test_trace_run_program_reads_the_model_folder(dtype, tmp_path):
             pos[e["id"]] += len(e["tokens"])
     err = worst_error(got, ref)
     assert err[0] <= TOL[dtype] and err[3] <= MEAN_TOL[dtype], err
+
+
+def test_the_serving_tools_take_the_design(tmp_path):
+    """kvmodel writes a random model folder from a configuration file, kvgen generates from it (greedy, against the plain
+    implementation on the folder's own tensors), kvbench serves a small workload with random weights of it."""
+    cfg_file = str(tmp_path / "r.json")
+    with open(cfg_file, "w") as f:
+        json.dump(cases.CONFIGS["R"], f)
+    d = str(tmp_path / "m")
+    tool = lambda name, *args: subprocess.run([sys.executable, os.path.join(ROOT, "bin", name), *args], capture_output=True,
+                                              text=True, timeout=300)
+    p = tool("kvmodel", "--out", d, "--config-json", cfg_file, "--weights-seed", "3", "--std", "0.08", "--norm-jitter", "0.1")
+    assert p.returncode == 0 and "Kasuvik" in p.stdout, p.stderr
+    prompt = [5, 17, 3, 100, 41, 77, 9]
+    p = tool("kvgen", "--model", d, "--dtype", "fp32", "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "10",
+             "--max-seq-len", "64", "--num-blocks", "16")
+    assert p.returncode == 0, p.stderr
+    t = plain.read_safetensors(os.path.join(d, "model.safetensors"))
+    toks = list(prompt)
+    for _ in range(10):
+        toks.append(int(np.argmax(plain.logits(cases.CONFIGS["R"], t, toks)[-1])))
+    assert [int(x) for x in p.stdout.split()] == toks[len(prompt):]
+    p = tool("kvbench", "--random-weights", "--config-json", cfg_file, "--dtype", "bf16", "--requests", "6", "--prompt-len", "9",
+             "--output-len", "5", "--max-seq-len", "64", "--num-blocks", "32", "--warmup", "1")
+    assert p.returncode == 0, p.stderr + p.stdout
