@@ -459,12 +459,6 @@ __global__ void __launch_bounds__(256)
 }
 
 
-// ------------------------------------------------------------------------- bfloat16 -> 32-bit
-__global__ void __launch_bounds__(256) widen_kernel(const uint16_t* __restrict__ in, float* __restrict__ out, size_t n) {
-  for (size_t i = blockIdx.x * size_t(blockDim.x) + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x)
-    out[i] = bf16_bits_to_float(in[i]);
-}
-
 }  // namespace kvcm
 
 using namespace kvcm;
@@ -472,15 +466,6 @@ using namespace kvcm;
 extern "C" {
 
 const char* kvcm_hip_last_error() { return g_hip_error.c_str(); }
-
-int kvcm_widen(const void* in, float* out, long long n, hipStream_t s) {
-  if (n == 0) return 0;
-  KVCM_REQUIRE(n > 0 && in != nullptr && out != nullptr, "widen: bad arguments");
-  const long long blocks = (n + 255) / 256;
-  widen_kernel<<<static_cast<unsigned>(blocks < 8192 ? blocks : 8192), 256, 0, s>>>(static_cast<const uint16_t*>(in), out,
-                                                                                   static_cast<size_t>(n));
-  return launch_status("widen");
-}
 
 int kvcm_embed_scaled(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, float factor,
                       hipStream_t s) {

@@ -42,6 +42,7 @@ struct Plan {
 std::mutex g_lock;
 hipblasLtHandle_t g_handle = nullptr;
 std::map<std::tuple<int, int, int, int, int, int>, Plan> g_plans;
+std::map<std::tuple<int, int, int, int, int, int>, Plan> g_plans_f32;      // the same products with a 32-bit result
 
 const char* status_name(hipblasStatus_t s) {
   switch (s) {
@@ -64,14 +65,14 @@ const char* status_name(hipblasStatus_t s) {
     }                                                                                \
   } while (0)
 
-int make_plan(Plan& p, int M, int N, int K, int ldx, int ldw, int ldo) {
+int make_plan(Plan& p, int M, int N, int K, int ldx, int ldw, int ldo, bool out_f32 = false) {
   KVCM_BLAS(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
   const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
   KVCM_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)));
   KVCM_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)));
   KVCM_BLAS(hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, K, N, ldw));   // W as stored, seen column-major
   KVCM_BLAS(hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16BF, K, M, ldx));   // X as stored, seen column-major
-  KVCM_BLAS(hipblasLtMatrixLayoutCreate(&p.c, HIP_R_16BF, N, M, ldo));   // the result, seen column-major
+  KVCM_BLAS(hipblasLtMatrixLayoutCreate(&p.c, out_f32 ? HIP_R_32F : HIP_R_16BF, N, M, ldo));   // the result, seen column-major
   hipblasLtMatmulPreference_t pref = nullptr;
   KVCM_BLAS(hipblasLtMatmulPreferenceCreate(&pref));
   const uint64_t cap = kWorkspaceBytes;
@@ -92,14 +93,15 @@ int make_plan(Plan& p, int M, int N, int K, int ldx, int ldw, int ldo) {
 }
 
 // The plan of a shape, made at its first use.  Call with g_lock held.
-int plan_for(Plan*& plan, int M, int N, int K, int ldx, int ldw, int ldo) {
+int plan_for(Plan*& plan, int M, int N, int K, int ldx, int ldw, int ldo, bool out_f32 = false) {
   if (g_handle == nullptr) KVCM_BLAS(hipblasLtCreate(&g_handle));
   const auto key = std::make_tuple(M, N, K, ldx, ldw, ldo);
-  auto it = g_plans.find(key);
-  if (it == g_plans.end()) {
+  auto& plans = out_f32 ? g_plans_f32 : g_plans;
+  auto it = plans.find(key);
+  if (it == plans.end()) {
     Plan p;
-    if (int rc = make_plan(p, M, N, K, ldx, ldw, ldo)) return rc;
-    it = g_plans.emplace(key, p).first;
+    if (int rc = make_plan(p, M, N, K, ldx, ldw, ldo, out_f32)) return rc;
+    it = plans.emplace(key, p).first;
   }
   plan = &it->second;   // entries of a std::map stay where they are
   return 0;
@@ -147,6 +149,38 @@ int kvcm_gemm_library(const void* X, const void* W, void* out, int M, int N, int
   }
   KVCM_REQUIRE(static_cast<long long>(algo_workspace) <= workspace_bytes && (algo_workspace == 0 || workspace != nullptr),
                "gemm_library: the algorithm needs %zu bytes of workspace, %lld were given", algo_workspace, workspace_bytes);
+  const float one = 1.0f, zero = 0.0f;
+  KVCM_BLAS(hipblasLtMatmul(g_handle, plan->desc, &one, W, plan->a, X, plan->b, &zero, out, plan->c, out, plan->c,
+                            &algo, workspace, algo_workspace, stream));
+  return 0;
+}
+
+// The same product with a 32-bit result (bfloat16 operands, 32-bit sums stored as they are), for consumers that
+// compute in 32-bit.  The heuristic's first choice; these plans are not tuned.  kvcm_gemm_library_f32out_plan makes
+// the shape's plan and tells whether the library has an algorithm for it (0: yes), outside any capture.
+int kvcm_gemm_library_f32out_plan(int M, int N, int K, int ldx, int ldw, int ldo) {
+  std::lock_guard<std::mutex> hold(g_lock);
+  Plan* plan = nullptr;
+  return plan_for(plan, M, N, K, ldx, ldw, ldo, true);
+}
+
+int kvcm_gemm_library_f32out(const void* X, const void* W, float* out, int M, int N, int K, int ldx, int ldw, int ldo,
+                             void* workspace, long long workspace_bytes, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  KVCM_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_library_f32out: bad sizes M=%d N=%d K=%d", M, N, K);
+  KVCM_REQUIRE(ldx >= K && ldw >= K && ldo >= N, "gemm_library_f32out: leading dimensions too small");
+  KVCM_REQUIRE(X != nullptr && W != nullptr && out != nullptr, "gemm_library_f32out: null operand");
+  Plan* plan = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t algo_workspace = 0;
+  {
+    std::lock_guard<std::mutex> hold(g_lock);
+    if (int rc = plan_for(plan, M, N, K, ldx, ldw, ldo, true)) return rc;
+    algo = plan->algo;
+    algo_workspace = plan->workspace;
+  }
+  KVCM_REQUIRE(static_cast<long long>(algo_workspace) <= workspace_bytes && (algo_workspace == 0 || workspace != nullptr),
+               "gemm_library_f32out: the algorithm needs %zu bytes of workspace, %lld were given", algo_workspace, workspace_bytes);
   const float one = 1.0f, zero = 0.0f;
   KVCM_BLAS(hipblasLtMatmul(g_handle, plan->desc, &one, W, plan->a, X, plan->b, &zero, out, plan->c, out, plan->c,
                             &algo, workspace, algo_workspace, stream));

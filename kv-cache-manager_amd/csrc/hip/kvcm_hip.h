@@ -84,6 +84,10 @@ int kvcm_gemm8_residual_norm(const void* X, int ldx, const void* W, int ldw, int
 long long kvcm_gemm_library_workspace_bytes();
 int kvcm_gemm_library(const void* X, const void* W, void* out, int M, int N, int K, int ldx, int ldw, int ldo,
                       void* workspace, long long workspace_bytes, hipStream_t stream);
+// the same with a 32-bit result; _plan: 0 when the library has an algorithm for the shape
+int kvcm_gemm_library_f32out_plan(int M, int N, int K, int ldx, int ldw, int ldo);
+int kvcm_gemm_library_f32out(const void* X, const void* W, float* out, int M, int N, int K, int ldx, int ldw, int ldo,
+                             void* workspace, long long workspace_bytes, hipStream_t stream);
 // Which algorithm of the library a shape runs: the heuristic's first choice until this has timed
 // candidates on the shape's own operands (mode 1: the heuristic's choices, a few milliseconds; mode 2:
 // every algorithm that supports the shape, at most max_seconds) and kept the fastest whose result
@@ -146,12 +150,11 @@ int kvcm_probe_phases(const void* weights, const long long* phase_bytes, int pha
 int kvcm_embed_scaled(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, float factor,
                       hipStream_t s);
 int kvcm_gated_act(const float* gate_up, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s);
-int kvcm_widen(const void* in, float* out, long long n, hipStream_t s);      // contiguous bfloat16 -> 32-bit
 // (norm_chain.hip) 32-bit RMS norms chained along a row: two branches combined, normed, added to the stream, the
 // stream normed again; the norm of every head with a weight and a sigmoid gate
-int kvcm_rmsnorm_chain(float* x, const float* a, const float* b, const float* wa, const float* wb, float combine,
-                       const float* w_post, const int* rows, const float* w_pre, void* out, int out_dtype, int R, int H,
-                       float eps, hipStream_t s);
+int kvcm_rmsnorm_chain(float* x, const float* a, int a_splits, const float* b, int b_splits, long long split_stride,
+                       const float* wa, const float* wb, float combine, const float* w_post, const int* rows,
+                       const float* w_pre, void* out, int out_dtype, int R, int H, float eps, hipStream_t s);
 int kvcm_head_norm_gate(const float* o, int ldo, const float* g, int ldg, const float* w, void* out, int out_dtype,
                         int ldout, int T, int heads, int d, float eps, hipStream_t s);
 // (short_conv.hip) a short causal convolution per channel over packed runs, its last inputs kept per sequence

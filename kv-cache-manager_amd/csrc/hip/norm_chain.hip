@@ -18,8 +18,9 @@ constexpr int kChainThreads = 256;
 
 template <class TO>
 __global__ void __launch_bounds__(kChainThreads)
-    rmsnorm_chain_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
-                         const float* __restrict__ wa, const float* __restrict__ wb, float combine,
+    rmsnorm_chain_kernel(float* __restrict__ x, const float* __restrict__ a, int a_splits, const float* __restrict__ b,
+                         int b_splits, size_t split_stride, const float* __restrict__ wa, const float* __restrict__ wb,
+                         float combine,
                          const float* __restrict__ w_post, const int* __restrict__ rows,
                          const float* __restrict__ w_pre, TO* __restrict__ out, int H, float eps, int write_back) {
   __shared__ float scratch[kChainThreads / kWave + 1];
@@ -29,12 +30,19 @@ __global__ void __launch_bounds__(kChainThreads)
   const float* ar = a ? a + size_t(src) * H : nullptr;
   const float* br = b ? b + size_t(src) * H : nullptr;
   const float inv_h = 1.0f / float(H);
+  // a branch is a finished tensor (splits 1) or the slices of a product that was split along K and not added up yet
+  // ([splits][T][H] floats): then the slices are added here, in their order
+  auto part = [&](const float* p, int splits, int i) {
+    float v = p[i];
+    for (int sl = 1; sl < splits; ++sl) v += p[size_t(sl) * split_stride + i];
+    return v;
+  };
 
   float inv_a = 0.f, inv_b = 0.f;
   if (br) {
     float sa = 0.f, sb = 0.f;
     for (int i = threadIdx.x; i < H; i += kChainThreads) {
-      const float u = ar[i], v = br[i];
+      const float u = part(ar, a_splits, i), v = part(br, b_splits, i);
       sa = fmaf(u, u, sa);
       sb = fmaf(v, v, sb);
     }
@@ -44,7 +52,7 @@ __global__ void __launch_bounds__(kChainThreads)
     inv_b = 1.0f / sqrtf(sb * inv_h + eps);
   }
   auto branch = [&](int i) {
-    return br ? combine * (ar[i] * inv_a * wa[i] + br[i] * inv_b * wb[i]) : ar[i];
+    return br ? combine * (part(ar, a_splits, i) * inv_a * wa[i] + part(br, b_splits, i) * inv_b * wb[i]) : part(ar, a_splits, i);
   };
   float inv_m = 0.f;
   if (ar) {
@@ -106,24 +114,26 @@ using namespace kvcm;
 
 extern "C" {
 
-// a, b: the branches [T, H] (b null: one branch, taken as it is; a null: nothing is added).  rows: source
+// a, b: the branches [T, H] (b null: one branch, taken as it is; a null: nothing is added), each finished (splits 1) or
+// the un-added slices of a split product, [splits][T][H] with split_stride = T * H floats between slices.  rows: source
 // rows of the R outputs (null: row r).  out null: only the addition.  The stream is updated in place
 // unless rows are gathered.
-int kvcm_rmsnorm_chain(float* x, const float* a, const float* b, const float* wa, const float* wb, float combine,
-                       const float* w_post, const int* rows, const float* w_pre, void* out, int out_dtype, int R, int H,
-                       float eps, hipStream_t s) {
+int kvcm_rmsnorm_chain(float* x, const float* a, int a_splits, const float* b, int b_splits, long long split_stride,
+                       const float* wa, const float* wb, float combine, const float* w_post, const int* rows,
+                       const float* w_pre, void* out, int out_dtype, int R, int H, float eps, hipStream_t s) {
   if (R == 0) return 0;
   KVCM_REQUIRE(R > 0 && H > 0 && x != nullptr, "rmsnorm_chain: bad sizes R=%d H=%d", R, H);
   KVCM_REQUIRE(!b || (a && wa && wb), "rmsnorm_chain: two branches need both outputs and both weights");
   KVCM_REQUIRE(!a || w_post, "rmsnorm_chain: an added output needs the weight of its norm");
   KVCM_REQUIRE(!out || w_pre, "rmsnorm_chain: a normed output needs its weight");
   KVCM_REQUIRE(out || (a && !rows), "rmsnorm_chain: nothing to do");
+  KVCM_REQUIRE(a_splits >= 1 && b_splits >= 1 && split_stride >= 0, "rmsnorm_chain: a branch has at least one slice");
   const int wb_flag = rows ? 0 : 1;
   if (!out || out_dtype == kF32)
-    rmsnorm_chain_kernel<float><<<R, kChainThreads, 0, s>>>(x, a, b, wa, wb, combine, w_post, rows, w_pre,
+    rmsnorm_chain_kernel<float><<<R, kChainThreads, 0, s>>>(x, a, a_splits, b, b_splits, static_cast<size_t>(split_stride), wa, wb, combine, w_post, rows, w_pre,
                                                              static_cast<float*>(out), H, eps, wb_flag);
   else if (out_dtype == kBF16)
-    rmsnorm_chain_kernel<bf16_t><<<R, kChainThreads, 0, s>>>(x, a, b, wa, wb, combine, w_post, rows, w_pre,
+    rmsnorm_chain_kernel<bf16_t><<<R, kChainThreads, 0, s>>>(x, a, a_splits, b, b_splits, static_cast<size_t>(split_stride), wa, wb, combine, w_post, rows, w_pre,
                                                               static_cast<bf16_t*>(out), H, eps, wb_flag);
   else KVCM_REQUIRE(false, "rmsnorm_chain: unknown output dtype %d", out_dtype);
   return launch_status("rmsnorm_chain");

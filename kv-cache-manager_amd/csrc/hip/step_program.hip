@@ -83,6 +83,7 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_gemm_f32),
     KVCM_ENTRY(kvcm_gemm_bf16),
     KVCM_ENTRY(kvcm_gemm_library),
+    KVCM_ENTRY(kvcm_gemm_library_f32out),
     KVCM_ENTRY(kvcm_gemm8),
     KVCM_ENTRY(kvcm_gemm8_residual_norm),
     KVCM_ENTRY(kvcm_attention_generic),
@@ -92,7 +93,6 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_sample),
     KVCM_ENTRY(kvcm_embed_scaled),
     KVCM_ENTRY(kvcm_gated_act),
-    KVCM_ENTRY(kvcm_widen),
     KVCM_ENTRY(kvcm_rmsnorm_chain),
     KVCM_ENTRY(kvcm_head_norm_gate),
     KVCM_ENTRY(kvcm_short_conv),

@@ -70,6 +70,8 @@ def _declare(lib):
     fn("kvcm_attention_decode", vp, i, vp, i, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, vp, C.c_longlong, vp)
     fn("kvcm_gemm_library", vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, vp)
     fn("kvcm_gemm_library_tuned", i, i, i, i, i, i)
+    fn("kvcm_gemm_library_f32out_plan", i, i, i, i, i, i)
+    fn("kvcm_gemm_library_f32out", vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, vp)
     fn("kvcm_gemm_library_tune", vp, vp, i, C.c_longlong, vp, i, i, i, i, i, i, vp, C.c_longlong, vp, i, C.c_double,
        C.POINTER(C.c_double), vp)
     fn("kvcm_probe_empty", i, i, vp)
@@ -87,8 +89,7 @@ def _declare(lib):
     fn("kvcm_gemm8_residual_norm", vp, i, vp, i, i, i, i, vp, vp, i, vp, vp, vp)
     fn("kvcm_embed_scaled", vp, vp, i, vp, i, i, i, f, vp)
     fn("kvcm_gated_act", vp, i, vp, i, i, i, i, i, vp)
-    fn("kvcm_widen", vp, vp, C.c_longlong, vp)
-    fn("kvcm_rmsnorm_chain", vp, vp, vp, vp, vp, f, vp, vp, vp, vp, i, i, i, f, vp)
+    fn("kvcm_rmsnorm_chain", vp, vp, i, vp, i, C.c_longlong, vp, vp, f, vp, vp, vp, vp, i, i, i, f, vp)
     fn("kvcm_head_norm_gate", vp, i, vp, i, vp, vp, i, i, i, i, i, f, vp)
     fn("kvcm_short_conv", vp, i, vp, vp, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_short_conv_state", vp, i, vp, vp, vp, vp, vp, vp, i, i, i, vp)
@@ -496,6 +497,17 @@ library_tuning_log = []          # (M, N, K, first choice's us, kept us, candida
 _library_ws = None
 
 
+_f32out_shapes = {}
+
+
+def _library_has_f32out(*shape):
+    """Does the library have an algorithm for this product with a 32-bit result?  Asked once per shape (the plan is
+    made then, outside any recorded launch)."""
+    if shape not in _f32out_shapes:
+        _f32out_shapes[shape] = lib().kvcm_gemm_library_f32out_plan(*shape) == 0
+    return _f32out_shapes[shape]
+
+
 def _library_workspace(device):
     """Device memory the vendor library's product may use (one buffer, kept: recorded steps hold its address)."""
     global _library_ws
@@ -548,6 +560,13 @@ def gemm(x, w, out, scratch=None, keep_partial=False, tuning=None):
         _call("kvcm_gemm_f32", _ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0), _stream())
         return out
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm operands must both be bfloat16")
+    if out.dtype == torch.float32 and out.is_contiguous() and _library_takes(M, N, K) and _library_has_f32out(
+            M, N, K, x.stride(0), w.stride(0), out.stride(0)):
+        # many rows, a 32-bit result: the library stores its 32-bit sums as they are
+        ws = _library_workspace(out.device)
+        _call("kvcm_gemm_library_f32out", _ptr(x), _ptr(w), _ptr(out), M, N, K, x.stride(0), w.stride(0), out.stride(0),
+              _ptr(ws), ws.numel(), _stream())
+        return out
     library = _library_takes(M, N, K) and out.dtype == torch.bfloat16 and out.is_contiguous()
     S = skinny_splits(M, N, K) if (not library and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
                                    and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0) else 0
@@ -946,20 +965,6 @@ def gated_act(gate_up, out, activation):
           GATE_ACTIVATIONS[activation], _stream())
 
 
-def widen(x, out):
-    """out (float32) = x (bfloat16), both contiguous and of one shape."""
-    _dev(x, out)
-    _need(x.dtype == torch.bfloat16 and out.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
-          and x.shape == out.shape, "widen takes a contiguous bfloat16 tensor and a float32 one of the same shape")
-    _call("kvcm_widen", _ptr(x), _ptr(out), x.numel(), _stream())
-    return out
-
-
-def library_takes(M, N, K):
-    """Does a bfloat16 product of this shape go to the vendor library (when its result is bfloat16)?"""
-    return bool(_library_takes(M, N, K))
-
-
 class NormedBranches:
     """A sublayer's output that is still to be normed and added to the residual stream:
     x += n(m) * w_post with m = a, or m = combine * (n(a) * wa + n(b) * wb) for two branches side by side
@@ -976,12 +981,20 @@ def rmsnorm_chain(x, eps, pending=None, weight=None, out=None, rows=None):
     _need(x.dtype == torch.float32 and x.is_contiguous() and x.is_cuda and x.dim() == 2, "x must be contiguous float32 [T, H]")
     T, H = x.shape
     a = b = wa = wb = wp = None
-    combine = 1.0
+    combine, a_splits, b_splits = 1.0, 1, 1
     if pending is not None:
         a, b, wa, wb, wp, combine = pending.a, pending.b, pending.wa, pending.wb, pending.w_post, pending.combine
-        for t, n in ((a, "a"), (b, "b")):
-            if t is not None:
-                _need(t.dtype == torch.float32 and t.is_contiguous() and t.shape == x.shape, f"branch {n} must match x")
+        # a branch may be the un-added slices of a split product (PartialSums [splits][T][H]): they are added here
+        if isinstance(a, PartialSums):
+            _need(a.rows == T and a.cols == H, "a branch's partial sums must match x")
+            a, a_splits = a.data, a.splits
+        elif a is not None:
+            _need(a.dtype == torch.float32 and a.is_contiguous() and a.shape == x.shape, "branch a must match x")
+        if isinstance(b, PartialSums):
+            _need(b.rows == T and b.cols == H, "a branch's partial sums must match x")
+            b, b_splits = b.data, b.splits
+        elif b is not None:
+            _need(b.dtype == torch.float32 and b.is_contiguous() and b.shape == x.shape, "branch b must match x")
         for t in (wa, wb, wp):
             _f32(t, "a norm weight", H)
     R = T
@@ -995,7 +1008,7 @@ def rmsnorm_chain(x, eps, pending=None, weight=None, out=None, rows=None):
             _need(R <= T, "x has fewer rows than the output")
     else:
         _need(pending is not None and rows is None, "rmsnorm_chain: nothing to do")
-    _call("kvcm_rmsnorm_chain", _ptr(x), _ptr(a), _ptr(b), _ptr(wa), _ptr(wb), combine, _ptr(wp), _ptr(rows), _ptr(weight),
+    _call("kvcm_rmsnorm_chain", _ptr(x), _ptr(a), a_splits, _ptr(b), b_splits, T * H, _ptr(wa), _ptr(wb), combine, _ptr(wp), _ptr(rows), _ptr(weight),
           _ptr(out), _DT[out.dtype] if out is not None else 0, R, H, float(eps), _stream())
     return out
 

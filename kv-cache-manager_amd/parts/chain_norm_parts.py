@@ -16,23 +16,20 @@ def f32_params(tensors):
     return {k: v.float().contiguous() for k, v in tensors.items()}
 
 
-def linear32(ctx, step, x, w, name, exact=False):
-    """x @ w^T as 32-bit rows for a consumer that computes in 32-bit.  The products of this package write their
-    32-bit sums as they are.  A many-row product that the vendor library would take runs there with a bfloat16
-    result that is widened afterwards (the library's kernels are several times faster at those shapes), unless
-    ``exact``: what enters a recurrence keeps its 32-bit sums at every row count.  (Few-row products stay split along K
-    with a second launch that adds the slices up: run unsplit they were slower by more than that launch costs,
-    0.71 -> 0.80 ms a decode step at width 2048, 1.25 -> 1.49 ms at 4096.)"""
-    ops = ctx.ops
-    M, N, K = x.shape[0], w.shape[0], w.shape[1]
-    if not exact and x.dtype == torch.bfloat16 and ops.library_takes(M, N, K):
-        half = _linear(ctx, step, x, w, name + "_h")
-        return ops.widen(half, step.ws(name, (M, N), torch.float32))
-    return _linear(ctx, step, x, w, name, dtype=torch.float32)
+def linear32(ctx, step, x, w, name, exact=False, keep_partial=False):
+    """x @ w^T as 32-bit rows for a consumer that computes in 32-bit: the product's 32-bit sums as they are, from this
+    package's kernels for few rows and from the vendor library's for many (``ops.gemm`` decides, as for every product).
+    ``exact`` marks what enters a recurrence; it runs the same way, since no path rounds the sums.  (Few-row products stay
+    split along K with a second launch that adds the slices up: run unsplit they were slower by more than that launch
+    costs, 0.71 -> 0.80 ms a decode step at width 2048, 1.25 -> 1.49 ms at 4096.)  ``keep_partial``: the product may
+    come back as ops.PartialSums for a consumer that adds the slices itself.  The chained norm can, and the parts do not
+    use it: one workgroup a row adding 8 + 8 slices in each of its passes takes longer than the launch it saves (a decode
+    step at width 2048 0.69 -> 0.96 ms)."""
+    return _linear(ctx, step, x, w, name, keep_partial=keep_partial, dtype=torch.float32)
 
 
 class BranchPair:
-    """Two sublayer outputs side by side, still to be combined as combine * (n(a) * wa + n(b) * wb)
+    """Two sublayer outputs (32-bit tensors, or the un-added slices of their last products) side by side, still to be combined as combine * (n(a) * wa + n(b) * wb)
     (n: division by the root mean square): what a mixer of two halves hands to the arrangement, which
     passes it on to the norm that adds it to the stream (one launch for all of it)."""
 
@@ -58,7 +55,7 @@ class ChainedRMSNorm(Norm):
         super().bind(f32_params(tensors))
 
     def pending(self, value):
-        """A sublayer's output (a 32-bit tensor, or a BranchPair) as what the stream's next norm adds:
+        """A sublayer's output (a 32-bit tensor, ops.PartialSums, or a BranchPair) as what the stream's next norm adds:
         x += n(value) * weight."""
         ops = self.ctx.ops
         if isinstance(value, BranchPair):

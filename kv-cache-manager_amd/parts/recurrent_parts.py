@@ -117,16 +117,9 @@ class GeneralDeltaMixer(_StatefulMixer):
         ops, p, w = self.ctx.ops, self.params, self.w
         heads, d = p["heads"], p["dim"]
         D, T = heads * d, step.rows
-        if h.dtype == torch.bfloat16 and ops.library_takes(T, 4 * D, h.shape[1]):
-            # many rows: r, k, v, g through the vendor library; what enters the recurrence's decay and removal rate keeps its sums
-            rkvg = linear32(self.ctx, step, h, w["w_proj"][:4 * D], "delta_rkvg")
-            rest = _linear(self.ctx, step, h, w["w_proj"][4 * D:], "delta_a_low", dtype=torch.float32)
-            r, k, v, g = (rkvg[:, i * D:(i + 1) * D] for i in range(4))
-            a, low = rest[:, :D], rest[:, D:]
-        else:
-            proj = linear32(self.ctx, step, h, w["w_proj"], "delta_proj", exact=True)
-            r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
-            low = proj[:, 5 * D:]
+        proj = linear32(self.ctx, step, h, w["w_proj"], "delta_proj", exact=True)
+        r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
+        low = proj[:, 5 * D:]
         decay, au, u = (step.ws(n, (T, D), torch.float32) for n in ("delta_w", "delta_au", "delta_u"))
         ops.delta_prepare(k, a, w["a_bias"], low, w["w2"], w["w0"], decay, au, u, heads, d, T)
         o = step.ws("delta_o", (T, D), torch.float32)

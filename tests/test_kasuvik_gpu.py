@@ -83,6 +83,21 @@ def test_chained_norms_against_the_plain_norm():
                 np.testing.assert_array_equal(xs.cpu().numpy(), x.astype(np.float32))
                 ops.rmsnorm_chain(xs, eps, pending=pending)
                 np.testing.assert_allclose(xs.cpu().numpy(), x + added, atol=2e-5)
+    # a branch that is still the slices of a split product: the norm adds them up itself
+    T, H = 3, 200
+    x, eps = rng.normal(size=(T, H)), 1e-6
+    sa, sb = rng.normal(size=(4, T, H)), rng.normal(size=(2, T, H))
+    wa, wb, wp, w = (1.0 + 0.2 * rng.normal(size=H) for _ in range(4))
+    a, b = sa.sum(0), sb.sum(0)
+    m = 0.5 * (plain.rms_norm(a, wa, eps) + plain.rms_norm(b, wb, eps))
+    slices = lambda t: ops.PartialSums(dev(t), t.shape[0], T, H, torch.empty(T, H, device=DEV))
+    for pending, added in ((ops.NormedBranches(slices(sa), dev(wp)), plain.rms_norm(a, wp, eps)),
+                           (ops.NormedBranches(slices(sa), dev(wp), slices(sb), dev(wa), dev(wb), 0.5), plain.rms_norm(m, wp, eps)),
+                           (ops.NormedBranches(dev(a), dev(wp), slices(sb), dev(wa), dev(wb), 0.5), plain.rms_norm(m, wp, eps))):
+        xs, out = dev(x), torch.empty(T, H, device=DEV)
+        ops.rmsnorm_chain(xs, eps, pending=pending, weight=dev(w), out=out)
+        np.testing.assert_allclose(xs.cpu().numpy(), x + added, atol=2e-5)
+        np.testing.assert_allclose(out.cpu().numpy(), plain.rms_norm(x + added, w, eps), atol=2e-5)
     # bfloat16 output: one rounding of the 32-bit result
     xs, out = dev(x), torch.empty(T, H, device=DEV, dtype=torch.bfloat16)
     ops.rmsnorm_chain(xs, eps, weight=dev(w), out=out)
@@ -164,7 +179,8 @@ def _pages(rng, tokens, B, nkv, d, dv, P, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [dict(nh=4, nkv=2, d=16, dv=24, rot=8, B=16, W=20, P=5), dict(nh=2, nkv=2, d=10, dv=6, rot=0, B=8, W=9, P=20),
                                    dict(nh=3, nkv=1, d=32, dv=72, rot=32, B=16, W=33, P=16), dict(nh=1, nkv=1, d=8, dv=8, rot=4, B=16, W=6, P=1),
-                                   dict(nh=2, nkv=1, d=64, dv=64, rot=64, B=32, W=0, P=0)])
+                                   dict(nh=2, nkv=1, d=64, dv=64, rot=64, B=32, W=0, P=0),
+                                   dict(nh=2, nkv=2, d=96, dv=136, rot=40, B=16, W=70, P=12)])
 def test_rotation_pages_pooled_blocks_and_attention(shape, dtype):
     """Rows written in portions through a shuffled page table; keys that decide the result placed just inside and
     just outside the window and in the newest seen and the first unseen block."""
@@ -225,7 +241,7 @@ def test_rotation_pages_pooled_blocks_and_attention(shape, dtype):
 def test_selective_scan_against_the_plain_recurrence():
     from kvcm_amd import ops
     rng = np.random.default_rng(5)
-    for C, N in ((40, 6), (70, 17), (9, 33), (130, 1)):
+    for C, N in ((40, 6), (70, 17), (9, 33), (130, 1), (20, 100)):
         lengths = (31, 2, 17)
         data = []
         for n in lengths:
