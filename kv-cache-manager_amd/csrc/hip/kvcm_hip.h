@@ -187,7 +187,8 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
 int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
                         const float* bc, int ldbc, int off_b, int off_c, const float* a_log, const float* dskip,
                         const float* z, int ldz, void* out, int ldo, float* state, const int* run_start,
-                        const int* seq_start, const int* state_slots, int S, int C, int N, int prepared, hipStream_t s);
+                        const int* seq_start, const int* state_slots, int S, int C, int N, int prepared, int chunk_len,
+                        int max_run, float* carry, long long carry_floats, int T, hipStream_t s);
 int kvcm_scan_prepare(float* dt, int lddt, const float* dt_bias, float* z, int ldz, int T, int C, hipStream_t s);
 int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, const float* a_bias, const float* low, int ldlow,
                        const float* w2t, int rank, const float* w0, float* w_out, float* au_out, float* u_out, int T, int heads,

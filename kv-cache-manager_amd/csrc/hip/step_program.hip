@@ -109,7 +109,7 @@ const Entry kEntries[] = {
 };
 #undef KVCM_ENTRY
 
-constexpr int kMaxArgs = 28;
+constexpr int kMaxArgs = 32;
 
 struct Launch {
   const Entry* entry;

@@ -99,7 +99,7 @@ def _declare(lib):
     fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp)
     fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
     fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, vp)
-    fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, i, vp)
     fn("kvcm_scan_prepare", vp, i, vp, vp, i, i, i, vp)
     fn("kvcm_delta_prepare", vp, i, vp, i, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_delta_scan", vp, i, vp, i, vp, i, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, vp)
@@ -1171,10 +1171,21 @@ def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_st
           d, dv, B, float(scale), int(window), int(P), E, _stream())
 
 
-def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, state, step, prepare=False):
+SCAN_PIECE = 128      # rows of a piece when long runs are walked in pieces
+
+
+def selective_scan_carry_floats(rows, seqs, C, N, piece=SCAN_PIECE):
+    """32-bit values of scratch that ``selective_scan(..., pieces=True)`` needs for a step of this shape."""
+    return (rows // piece + seqs + 1) * C * (N + 1)
+
+
+def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, state, step, prepare=False, carry=None):
     """The selective scan of the step's runs (csrc/hip/selective_scan.hip).  x, out [T, C] in the compute dtype;
     dt_lin [T, C], bc rows with B at off_b and C at off_c, z rows: 32-bit; state [slots, C, N].  ``prepare``: the step
-    sizes and gates of all rows are made first, in place in dt_lin and z, by a launch of their own (pays for long runs)."""
+    sizes and gates of all rows are made first, in place in dt_lin and z, by a launch of their own (pays for long runs).
+    ``carry`` (float32 scratch of ``selective_scan_carry_floats``; needs ``prepare``): runs are walked in pieces of
+    SCAN_PIECE rows, all pieces at once: each from zero, then the states that enter the pieces (a short walk over the
+    pieces' ends), then each again from its entering state.  The sums are the token-by-token ones in another order."""
     C, N = a_log.shape
     _rows2d(x, "x")
     _rows2d(out, "out")
@@ -1187,11 +1198,16 @@ def selective_scan(x, dt_lin, dt_bias, bc, off_b, off_c, a_log, dskip, z, out, s
     _f32(dskip, "dskip", C)
     _need(state.dtype == torch.float32 and state.is_contiguous() and state.is_cuda and tuple(state.shape[1:]) == (C, N),
           "state must be float32 [slots, C, N]")
+    if carry is not None:
+        _need(prepare and carry.dtype == torch.float32 and carry.is_contiguous() and carry.is_cuda
+              and carry.numel() >= selective_scan_carry_floats(out.shape[0], step.seqs, C, N), "the scratch for the pieces is too small")
     if prepare:
         _call("kvcm_scan_prepare", _ptr(dt_lin), dt_lin.stride(0), _ptr(dt_bias), _ptr(z), z.stride(0), out.shape[0], C, _stream())
     _call("kvcm_selective_scan", _ptr(x), _DT[x.dtype], x.stride(0), _ptr(dt_lin), dt_lin.stride(0), _ptr(dt_bias), _ptr(bc),
           bc.stride(0), off_b, off_c, _ptr(a_log), _ptr(dskip), _ptr(z), z.stride(0), _ptr(out), out.stride(0), _ptr(state),
-          _ptr(step.run_start), _ptr(step.seq_start), _ptr(step.state_slots), step.seqs, C, N, 1 if prepare else 0, _stream())
+          _ptr(step.run_start), _ptr(step.seq_start), _ptr(step.state_slots), step.seqs, C, N, 1 if prepare else 0,
+          SCAN_PIECE if carry is not None else 0, step.max_run, _ptr(carry), carry.numel() if carry is not None else 0,
+          out.shape[0], _stream())
     return out
 
 

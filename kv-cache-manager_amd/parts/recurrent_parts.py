@@ -71,8 +71,12 @@ class SelectiveScanMixer(_StatefulMixer):
         bc = _linear(self.ctx, step, x, w["w_x"][R:], "scan_bc", dtype=torch.float32)
         dt = linear32(self.ctx, step, low, w["w_dt"], "scan_dt", exact=True)
         y = step.ws("scan_y", (step.rows, C))
+        # runs of some length: step sizes and gates made ahead; long runs: walked in pieces, all pieces at once
+        carry = None
+        if step.max_run >= 4 * ops.SCAN_PIECE:
+            carry = step.flat("scan_carry", ops.selective_scan_carry_floats(max(step.rows, step.limits.max_tokens), step.limits.max_seqs, C, N))
         ops.selective_scan(x, dt, w["dt_bias"], bc, 0, N, w["a_log"], w["d_skip"], xz[:, C:], y, self.state("scan"), step,
-                           prepare=step.max_run >= 16)
+                           prepare=step.max_run >= 16, carry=carry)
         return linear32(self.ctx, step, y, w["w_o"], "scan_out")
 
 

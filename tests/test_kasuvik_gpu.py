@@ -257,6 +257,7 @@ def test_selective_scan_against_the_plain_recurrence():
             step = Step(runs)
             cat = lambda i: dev(np.concatenate([data[s][i][p:p + n] for s, p, n in runs]))
             out = torch.empty(step.rows, C, device=DEV)
+            step.max_run = max(n for _, _, n in runs)
             ops.selective_scan(cat(0), cat(2), dev(db), cat(3), 3, 3 + N, dev(a_log), dev(dsk), cat(1), out, state, step)
             r = 0
             for s, p, n in runs:
@@ -264,6 +265,34 @@ def test_selective_scan_against_the_plain_recurrence():
                 r += n
         for s in range(len(lengths)):
             np.testing.assert_allclose(got[s], want[s], atol=3e-5 * max(1.0, np.abs(want[s]).max()))
+
+
+def test_selective_scan_of_long_runs_in_pieces():
+    """Runs walked in pieces of 128 rows, all pieces at once, in steps that hold several sequences whose runs start
+    anywhere, with the state carried from step to step: against the plain token-by-token recurrence."""
+    from kvcm_amd import ops
+    rng = np.random.default_rng(15)
+    C, N, lengths = 70, 17, (900, 131, 1, 640)
+    data = [(rng.normal(size=(n, C)), rng.normal(size=(n, C)), rng.normal(size=(n, C)) - 1.0, rng.normal(size=(n, 2 * N))) for n in lengths]
+    a_log, dsk, db = np.log(rng.uniform(0.3, 4.0, size=(C, N))), rng.normal(size=C), rng.normal(size=C)
+    want = [plain.selective_scan(x, plain.softplus(dtl + db), -np.exp(a_log), bc[:, :N], bc[:, N:], dsk) * plain.silu(z)
+            for x, z, dtl, bc in data]
+    state = torch.full((len(lengths), C, N), 5.0, device=DEV)
+    got = [np.zeros((n, C)) for n in lengths]
+    plan = [[(0, 0, 517), (1, 0, 131), (3, 0, 1)], [(3, 1, 639), (2, 0, 1), (0, 517, 130)], [(0, 647, 253)]]
+    for runs in plan:
+        step = Step(runs)
+        step.max_run = max(n for _, _, n in runs)
+        cat = lambda i: dev(np.concatenate([data[s][i][p:p + n] for s, p, n in runs]))
+        out = torch.empty(step.rows, C, device=DEV)
+        carry = torch.full((ops.selective_scan_carry_floats(step.rows, step.seqs, C, N),), float("nan"), device=DEV)
+        ops.selective_scan(cat(0), cat(2), dev(db), cat(3), 0, N, dev(a_log), dev(dsk), cat(1), out, state, step, prepare=True, carry=carry)
+        r = 0
+        for s, p, n in runs:
+            got[s][p:p + n] = out[r:r + n].cpu().numpy()
+            r += n
+    for s in range(len(lengths)):
+        np.testing.assert_allclose(got[s], want[s], atol=3e-5 * max(1.0, np.abs(want[s]).max()))
 
 
 def test_delta_rule_against_the_plain_recurrence():
