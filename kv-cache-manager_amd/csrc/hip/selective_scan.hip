@@ -19,6 +19,13 @@
 
 namespace kvcm {
 
+// exp of a decay's exponent for a walk whose inputs and outputs are stored as T: exact for float; for bfloat16 the
+// hardware's exp2 (about one unit in the last place of a 32-bit value, a tenth of the instructions), which is far
+// inside what the storage type keeps of x and of the result.
+template <class T> __device__ __forceinline__ float decay_exp(float v);
+template <> __device__ __forceinline__ float decay_exp<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ float decay_exp<bf16_t>(float v) { return __builtin_amdgcn_exp2f(1.44269504088896341f * v); }
+
 constexpr int kScanAhead = 4;      // tokens whose inputs are on their way while the ones before are computed
 
 template <class T, int LPC, int NPL>
@@ -75,11 +82,12 @@ __global__ void __launch_bounds__(kWave)
       const int r = first + u < r1 ? first + u : r1 - 1;
       dtv[into][u] = dt_lin[size_t(r) * lddt + c];
       xv[into][u] = load_f(x + size_t(r) * ldx + c);
-      zv[into][u] = z[size_t(r) * ldz + c];
 #pragma unroll
-      for (int k = 0; k < NPL; ++k) {
-        bv[into][u][k] = bc[size_t(r) * ldbc + off_b + nidx[k]];
-        cv[into][u][k] = bc[size_t(r) * ldbc + off_c + nidx[k]];
+      for (int k = 0; k < NPL; ++k) bv[into][u][k] = bc[size_t(r) * ldbc + off_b + nidx[k]];
+      if (phase != 1) {      // (the same for every lane) the pass that only wants the state needs neither the gate nor C
+        zv[into][u] = z[size_t(r) * ldz + c];
+#pragma unroll
+        for (int k = 0; k < NPL; ++k) cv[into][u][k] = bc[size_t(r) * ldbc + off_c + nidx[k]];
       }
     }
   };
@@ -95,11 +103,12 @@ __global__ void __launch_bounds__(kWave)
         float y = 0.f;
 #pragma unroll
         for (int k = 0; k < NPL; ++k) {
-          const float sn = fmaf(expf(dt * A[k]), S[k], dx * bv[from][u][k]);
+          const float sn = fmaf(decay_exp<T>(dt * A[k]), S[k], dx * bv[from][u][k]);
           S[k] = has[k] ? sn : 0.f;
-          y = fmaf(S[k], cv[from][u][k], y);
         }
         if (phase == 1) continue;      // only the state is wanted
+#pragma unroll
+        for (int k = 0; k < NPL; ++k) y = fmaf(S[k], cv[from][u][k], y);
         y = group_sum<LPC>(y);
         if (owns && sub == 0) {
           y = fmaf(dk, xv[from][u], y);
