@@ -20,7 +20,7 @@
 
 namespace kvcm {
 
-constexpr int kDeltaTile = 8;      // tokens staged at once
+// (tokens staged at once: a template parameter of the walk, fewer for the largest key size so that the values on their way fit the registers)
 
 // one wave per (row, head).  The decay's logit is a two-step projection whose second step runs here in 32-bit:
 // w_lin[c] = sum_j w2[c, j] * tanh(low[j]), low = the first step's output (rank values a row); w2 comes transposed,
@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(256)
 // sequence; the key dimension of a column is spread over G lanes (IPT = DKP / G entries each, DKP: dk padded
 // with zeros), so a token costs a lane IPT multiply-adds for u^T S, a sum across its G lanes, 3 IPT
 // multiply-adds for the update, IPT for o and another sum across the lanes.
-template <int DKP, int G>
+template <int DKP, int G, int TILE>
 __global__ void __launch_bounds__(256)
     delta_scan_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
                       const float* __restrict__ v, int ldv, const float* __restrict__ w, const float* __restrict__ au,
@@ -72,8 +72,8 @@ __global__ void __launch_bounds__(256)
                       const int* __restrict__ run_start, const int* __restrict__ seq_start,
                       const int* __restrict__ state_slots, int heads, int dk, int dv, int col_blocks) {
   constexpr int IPT = DKP / G, CB = 256 / G, W = 5 * DKP + CB;
-  constexpr int PF = (kDeltaTile * W + 255) / 256;
-  __shared__ __attribute__((aligned(16))) float tile[kDeltaTile][W];      // per token: r, k, w, a*u, u (zero beyond dk), v of these columns
+  constexpr int PF = (TILE * W + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float tile[TILE][W];      // per token: r, k, w, a*u, u (zero beyond dk), v of these columns
   const int s = blockIdx.y, head = blockIdx.x / col_blocks, cb = blockIdx.x % col_blocks;
   const int g = threadIdx.x % G, j = cb * CB + threadIdx.x / G;
   const int r0 = run_start[s], r1 = run_start[s + 1];
@@ -106,7 +106,7 @@ __global__ void __launch_bounds__(256)
       const bool vector = off < 5 * DKP;
       const int which = off / DKP, i = off % DKP;
       const int jj = cb * CB + (off - 5 * DKP);
-      const bool ok = t < kDeltaTile && t0 + t < r1 && (vector ? i < dk : jj < dv);
+      const bool ok = t < TILE && t0 + t < r1 && (vector ? i < dk : jj < dv);
       const size_t col = size_t(head) * dk + (i < dk ? i : dk - 1);
       const size_t vcol = size_t(head) * dv + ((jj >= 0 && jj < dv) ? jj : 0);
       const float* src = !vector     ? v + size_t(row) * ldv + vcol
@@ -123,16 +123,16 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int q = 0; q < PF; ++q) {
       const int e = threadIdx.x + q * 256;
-      if (e < kDeltaTile * W) tile[e / W][e % W] = pf[q];
+      if (e < TILE * W) tile[e / W][e % W] = pf[q];
     }
   };
   request(r0);
   stage();
   __syncthreads();
-  for (int t0 = r0; t0 < r1; t0 += kDeltaTile) {
-    const int nt = r1 - t0 < kDeltaTile ? r1 - t0 : kDeltaTile;
-    const bool more = t0 + kDeltaTile < r1;
-    if (more) request(t0 + kDeltaTile);
+  for (int t0 = r0; t0 < r1; t0 += TILE) {
+    const int nt = r1 - t0 < TILE ? r1 - t0 : TILE;
+    const bool more = t0 + TILE < r1;
+    if (more) request(t0 + TILE);
     for (int t = 0; t < nt; ++t) {
       const float* tv = tile[t];
       const float vj = tv[5 * DKP + threadIdx.x / G];
@@ -196,21 +196,22 @@ int kvcm_delta_scan(const float* r, int ldr, const float* k, int ldk, const floa
                     const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s) {
   if (S == 0) return 0;
   KVCM_REQUIRE(S > 0 && heads > 0 && dk > 0 && dv > 0, "delta_scan: bad sizes S=%d heads=%d dk=%d dv=%d", S, heads, dk, dv);
-  KVCM_REQUIRE(dk <= 128, "delta_scan: a key size of %d is not supported (up to 128)", dk);
+  KVCM_REQUIRE(dk <= 256, "delta_scan: a key size of %d is not supported (up to 256)", dk);
   KVCM_REQUIRE(static_cast<long long>(heads) * ((dv + 31) / 32) < (1ll << 31), "delta_scan: too many heads");
   KVCM_REQUIRE(S <= 65535, "delta_scan: too many sequences for one launch (%d)", S);
   KVCM_REQUIRE(ldr >= heads * dk && ldk >= heads * dk && ldv >= heads * dv && ldo >= heads * dv, "delta_scan: row strides too small");
-#define KVCM_DELTA(DKP, G)                                                                                            \
+#define KVCM_DELTA(DKP, G, TILE)                                                                                            \
   {                                                                                                                    \
     const int col_blocks = (dv + 256 / G - 1) / (256 / G);                                                             \
-    delta_scan_kernel<DKP, G><<<dim3(heads * col_blocks, S), 256, 0, s>>>(r, ldr, k, ldk, v, ldv, w, au, u, o, ldo, state, \
+    delta_scan_kernel<DKP, G, TILE><<<dim3(heads * col_blocks, S), 256, 0, s>>>(r, ldr, k, ldk, v, ldv, w, au, u, o, ldo, state, \
                                                                           run_start, seq_start, state_slots, heads, dk, dv, \
                                                                           col_blocks);                                  \
   }
-  if (dk <= 16) KVCM_DELTA(16, 2)
-  else if (dk <= 32) KVCM_DELTA(32, 4)
-  else if (dk <= 64) KVCM_DELTA(64, 8)
-  else KVCM_DELTA(128, 8)
+  if (dk <= 16) KVCM_DELTA(16, 2, 8)
+  else if (dk <= 32) KVCM_DELTA(32, 4, 8)
+  else if (dk <= 64) KVCM_DELTA(64, 8, 8)
+  else if (dk <= 128) KVCM_DELTA(128, 8, 8)
+  else KVCM_DELTA(256, 16, 2)
 #undef KVCM_DELTA
   return launch_status("delta_scan");
 }

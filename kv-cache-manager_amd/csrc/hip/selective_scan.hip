@@ -190,7 +190,8 @@ int launch_scan(const void* x, int ldx, const float* dt_lin, int lddt, const flo
   else if (N <= 16) KVCM_SCAN(16, 1);
   else if (N <= 32) KVCM_SCAN(32, 1);
   else if (N <= 64) KVCM_SCAN(64, 1);
-  else KVCM_SCAN(64, 2);
+  else if (N <= 128) KVCM_SCAN(64, 2);
+  else KVCM_SCAN(64, 4);
 #undef KVCM_SCAN
   return launch_status("selective_scan");
 }
@@ -211,7 +212,7 @@ extern "C" int kvcm_selective_scan(const void* x, int dtype, int ldx, const floa
                                    int chunk_len, int max_run, float* carry, long long carry_floats, int T, hipStream_t s) {
   if (S == 0) return 0;
   KVCM_REQUIRE(S > 0 && C > 0 && N > 0, "selective_scan: bad sizes S=%d C=%d N=%d", S, C, N);
-  KVCM_REQUIRE(N <= 128, "selective_scan: a state of %d per channel is not supported (up to 128)", N);
+  KVCM_REQUIRE(N <= 256, "selective_scan: a state of %d per channel is not supported (up to 256)", N);
   KVCM_REQUIRE(S <= 65535, "selective_scan: too many sequences for one launch (%d)", S);
   KVCM_REQUIRE(ldx >= C && lddt >= C && ldz >= C && ldo >= C && off_b >= 0 && off_c >= 0 && ldbc >= off_b + N &&
                    ldbc >= off_c + N, "selective_scan: row strides too small");

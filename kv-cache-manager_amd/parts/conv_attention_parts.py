@@ -8,7 +8,6 @@ import torch
 from ..registry import MIXERS, POSITIONS
 from .base import KVCacheNeed, Mixer, ParamSpec, PartSpec, PositionEncoding, StateNeed
 from .chain_norm_parts import BranchPair, f32_params, linear32
-from .llama_parts import _linear
 
 
 @POSITIONS.register("rotary_pairs")

@@ -241,7 +241,7 @@ def test_rotation_pages_pooled_blocks_and_attention(shape, dtype):
 def test_selective_scan_against_the_plain_recurrence():
     from kvcm_amd import ops
     rng = np.random.default_rng(5)
-    for C, N in ((40, 6), (70, 17), (9, 33), (130, 1), (20, 100)):
+    for C, N in ((40, 6), (70, 17), (9, 33), (130, 1), (20, 100), (5, 200)):
         lengths = (31, 2, 17)
         data = []
         for n in lengths:
@@ -298,7 +298,7 @@ def test_selective_scan_of_long_runs_in_pieces():
 def test_delta_rule_against_the_plain_recurrence():
     from kvcm_amd import ops
     rng = np.random.default_rng(6)
-    for heads, d, rank in ((3, 16, 8), (1, 24, 5), (2, 48, 16), (2, 70, 3)):
+    for heads, d, rank in ((3, 16, 8), (1, 24, 5), (2, 48, 16), (2, 70, 3), (1, 136, 4)):
         D, lengths, eps = heads * d, (37, 1, 14), 1e-5
         seqs = []
         for n in lengths:
