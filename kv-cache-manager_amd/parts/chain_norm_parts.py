@@ -16,14 +16,14 @@ def f32_params(tensors):
     return {k: v.float().contiguous() for k, v in tensors.items()}
 
 
-def linear32(ctx, step, x, w, name, exact=False, keep_partial=False):
+def linear32(ctx, step, x, w, name, keep_partial=False):
     """x @ w^T as 32-bit rows for a consumer that computes in 32-bit: the product's 32-bit sums as they are, from this
-    package's kernels for few rows and from the vendor library's for many (``ops.gemm`` decides, as for every product).
-    ``exact`` marks what enters a recurrence; it runs the same way, since no path rounds the sums.  (Few-row products stay
+    package's kernels for few rows and from the vendor library's for many (``ops.gemm`` decides, as for every product);
+    no path rounds the sums, so what enters a recurrence is as exact at one row as at thousands.  Few-row products stay
     split along K with a second launch that adds the slices up: run unsplit they were slower by more than that launch
-    costs, 0.71 -> 0.80 ms a decode step at width 2048, 1.25 -> 1.49 ms at 4096.)  ``keep_partial``: the product may
-    come back as ops.PartialSums for a consumer that adds the slices itself.  The chained norm can, and the parts do not
-    use it: one workgroup a row adding 8 + 8 slices in each of its passes takes longer than the launch it saves (a decode
+    costs (a decode step at width 2048 0.71 -> 0.80 ms, at 4096 1.25 -> 1.49 ms).  ``keep_partial``: the product may come
+    back as ops.PartialSums for a consumer that adds the slices itself.  The chained norm can, and the parts do not use
+    it: one workgroup a row adding 8 + 8 slices in each of its passes takes longer than the launch it saves (a decode
     step at width 2048 0.69 -> 0.96 ms)."""
     return _linear(ctx, step, x, w, name, keep_partial=keep_partial, dtype=torch.float32)
 

@@ -68,8 +68,8 @@ class SelectiveScanMixer(_StatefulMixer):
             ops.short_conv_state(xz, conv_state, step, K)
         # the step size's low-rank input feeds a product (compute dtype); B and C enter the recurrence (32-bit)
         low = _linear(self.ctx, step, x, w["w_x"][:R], "scan_dt_low")
-        bc = _linear(self.ctx, step, x, w["w_x"][R:], "scan_bc", dtype=torch.float32)
-        dt = linear32(self.ctx, step, low, w["w_dt"], "scan_dt", exact=True)
+        bc = linear32(self.ctx, step, x, w["w_x"][R:], "scan_bc")
+        dt = linear32(self.ctx, step, low, w["w_dt"], "scan_dt")
         y = step.ws("scan_y", (step.rows, C))
         # runs of some length: step sizes and gates made ahead; long runs: walked in pieces, all pieces at once
         carry = None
@@ -121,7 +121,7 @@ class GeneralDeltaMixer(_StatefulMixer):
         ops, p, w = self.ctx.ops, self.params, self.w
         heads, d = p["heads"], p["dim"]
         D, T = heads * d, step.rows
-        proj = linear32(self.ctx, step, h, w["w_proj"], "delta_proj", exact=True)
+        proj = linear32(self.ctx, step, h, w["w_proj"], "delta_proj")
         r, k, v, g, a = (proj[:, i * D:(i + 1) * D] for i in range(5))
         low = proj[:, 5 * D:]
         decay, au, u = (step.ws(n, (T, D), torch.float32) for n in ("delta_w", "delta_au", "delta_u"))
