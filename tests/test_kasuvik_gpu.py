@@ -441,6 +441,23 @@ def test_32bit_logits_do_not_depend_on_cut_batch_or_pages(models, name):
             np.testing.assert_allclose(other[rid], whole[rid], atol=2e-5, rtol=0)
 
 
+@pytest.mark.parametrize("case", [("P", "float32"), ("R", "bfloat16"), ("Q", "bfloat16")])
+def test_steps_replayed_from_recorded_launch_lists(models, case):
+    """Every part says it is capturable: a step's shape (rows, wanted rows and longest run padded to multiples of 64)
+    is recorded once as a list of launches and replayed with only the step's metadata changed; padding rows and padding
+    sequences must leave pages and states alone."""
+    from kvcm_amd.engine.replay import TraceReplayer
+    _, reqs, ref, raw, _ = models(*case)
+    cfg, tensors = cases.tensors_for(raw, seed=len(case[0]) + sum(map(ord, case[0])))
+    rp = TraceReplayer(None, case[1], max_tokens=tokens_needed(reqs, 3), block_size=cases.BLOCK_SIZE[case[0]], max_live=3,
+                       architecture="Kasuvik", model_config=cfg, tensors=tensors, use_programs=True)
+    assert rp.programs is not None
+    for steps in (schedule_mixed(reqs, seed=5, max_live=3), schedule_tail_singly(reqs, tail=20)):
+        err = worst_error(replay(rp, steps, reqs), ref)
+        assert err[0] <= TOL[case[1]] and err[3] <= MEAN_TOL[case[1]], err
+    assert rp.steps_replayed > 50
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_far_beyond_windows_and_blocks(models, dtype):
     rp, _, _, raw, t = models("P", dtype)
@@ -489,6 +506,7 @@ def test_greedy_generation_through_the_engine(name, tmp_path):
     for chunk in (0, 8):
         eng = Engine(d, EngineConfig(dtype="float32", block_size=cases.BLOCK_SIZE[name], max_seq_len=128, num_blocks=40,
                                      max_num_seqs=3, max_batched_tokens=64, prefill_chunk=chunk))
+        assert eng.recorded is not None          # steps are recorded and replayed, decode steps as graphs: as for Llama
         got = eng.generate(prompts, new)
         assert got == want, f"prefill_chunk={chunk}"
 
