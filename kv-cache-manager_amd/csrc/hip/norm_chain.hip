@@ -84,6 +84,95 @@ __global__ void __launch_bounds__(kChainThreads)
   }
 }
 
+// The same chain for rows whose length is a multiple of 4 and at most 1024 * G (G groups of four values a thread):
+// the branches' and the stream's values of a row are read once, 16 bytes a load, and stay in registers through all
+// stages, so the row costs one trip to memory instead of one per stage.  Which of the two kernels runs depends on the
+// row length (and on whether a branch is still in slices) only, never on the batch.
+template <class TO, int G>
+__global__ void __launch_bounds__(kChainThreads)
+    rmsnorm_chain_rows_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
+                              const float* __restrict__ wa, const float* __restrict__ wb, float combine,
+                              const float* __restrict__ w_post, const int* __restrict__ rows,
+                              const float* __restrict__ w_pre, TO* __restrict__ out, int H, float eps, int write_back) {
+  __shared__ float scratch[kChainThreads / kWave + 1];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* xr = x + size_t(src) * H;
+  const float inv_h = 1.0f / float(H);
+  float xv[G][4], av[G][4], bv[G][4];
+  bool in[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int i = (g * kChainThreads + threadIdx.x) * 4;
+    in[g] = i < H;
+    const int ic = in[g] ? i : 0;
+    const float4 vx = *reinterpret_cast<const float4*>(xr + ic);
+    xv[g][0] = vx.x; xv[g][1] = vx.y; xv[g][2] = vx.z; xv[g][3] = vx.w;
+    if (a) {
+      const float4 va = *reinterpret_cast<const float4*>(a + size_t(src) * H + ic);
+      av[g][0] = va.x; av[g][1] = va.y; av[g][2] = va.z; av[g][3] = va.w;
+    }
+    if (b) {
+      const float4 vb = *reinterpret_cast<const float4*>(b + size_t(src) * H + ic);
+      bv[g][0] = vb.x; bv[g][1] = vb.y; bv[g][2] = vb.z; bv[g][3] = vb.w;
+    }
+  }
+  if (b) {
+    float sa = 0.f, sb = 0.f;
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (in[g]) {
+          sa = fmaf(av[g][e], av[g][e], sa);
+          sb = fmaf(bv[g][e], bv[g][e], sb);
+        }
+    sa = block_sum<kChainThreads>(sa, scratch);
+    sb = block_sum<kChainThreads>(sb, scratch);
+    const float inv_a = 1.0f / sqrtf(sa * inv_h + eps), inv_b = 1.0f / sqrtf(sb * inv_h + eps);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int i = in[g] ? (g * kChainThreads + threadIdx.x) * 4 : 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) av[g][e] = combine * (av[g][e] * inv_a * wa[i + e] + bv[g][e] * inv_b * wb[i + e]);
+    }
+  }
+  if (a) {
+    float sm = 0.f;
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (in[g]) sm = fmaf(av[g][e], av[g][e], sm);
+    sm = block_sum<kChainThreads>(sm, scratch);
+    const float inv_m = 1.0f / sqrtf(sm * inv_h + eps);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int i = in[g] ? (g * kChainThreads + threadIdx.x) * 4 : 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) xv[g][e] += av[g][e] * inv_m * w_post[i + e];
+      if (in[g] && write_back) *reinterpret_cast<float4*>(xr + i) = float4{xv[g][0], xv[g][1], xv[g][2], xv[g][3]};
+    }
+  }
+  if (!out) return;
+  float sx = 0.f;
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (in[g]) sx = fmaf(xv[g][e], xv[g][e], sx);
+  sx = block_sum<kChainThreads>(sx, scratch);
+  const float inv_x = 1.0f / sqrtf(sx * inv_h + eps);
+  TO* o = out + size_t(r) * H;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    if (!in[g]) continue;
+    const int i = (g * kChainThreads + threadIdx.x) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) store_f(o + i + e, xv[g][e] * inv_x * w_pre[i + e]);
+  }
+}
+
 // out[r, h, :] = n(o[r, h, :]) * w[h, :] * sigmoid(g[r, h, :]): the norm of every head on its own, a
 // plain weight over all heads, and a gate.  One wave per (row, head).
 template <class TO>
@@ -129,13 +218,25 @@ int kvcm_rmsnorm_chain(float* x, const float* a, int a_splits, const float* b, i
   KVCM_REQUIRE(out || (a && !rows), "rmsnorm_chain: nothing to do");
   KVCM_REQUIRE(a_splits >= 1 && b_splits >= 1 && split_stride >= 0, "rmsnorm_chain: a branch has at least one slice");
   const int wb_flag = rows ? 0 : 1;
-  if (!out || out_dtype == kF32)
-    rmsnorm_chain_kernel<float><<<R, kChainThreads, 0, s>>>(x, a, a_splits, b, b_splits, static_cast<size_t>(split_stride), wa, wb, combine, w_post, rows, w_pre,
-                                                             static_cast<float*>(out), H, eps, wb_flag);
-  else if (out_dtype == kBF16)
-    rmsnorm_chain_kernel<bf16_t><<<R, kChainThreads, 0, s>>>(x, a, a_splits, b, b_splits, static_cast<size_t>(split_stride), wa, wb, combine, w_post, rows, w_pre,
-                                                              static_cast<bf16_t*>(out), H, eps, wb_flag);
-  else KVCM_REQUIRE(false, "rmsnorm_chain: unknown output dtype %d", out_dtype);
+  KVCM_REQUIRE(!out || out_dtype == kF32 || out_dtype == kBF16, "rmsnorm_chain: unknown output dtype %d", out_dtype);
+  const bool f32 = !out || out_dtype == kF32;
+  auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (a_splits == 1 && b_splits == 1 && H % 4 == 0 && H <= 8192 && aligned(x) && aligned(a) && aligned(b)) {
+#define KVCM_CHAIN_ROWS(TO, G)                                                                                     \
+  rmsnorm_chain_rows_kernel<TO, G><<<R, kChainThreads, 0, s>>>(x, a, b, wa, wb, combine, w_post, rows, w_pre,      \
+                                                               static_cast<TO*>(out), H, eps, wb_flag)
+    if (H <= 2048) { if (f32) KVCM_CHAIN_ROWS(float, 2); else KVCM_CHAIN_ROWS(bf16_t, 2); }
+    else if (H <= 4096) { if (f32) KVCM_CHAIN_ROWS(float, 4); else KVCM_CHAIN_ROWS(bf16_t, 4); }
+    else { if (f32) KVCM_CHAIN_ROWS(float, 8); else KVCM_CHAIN_ROWS(bf16_t, 8); }
+#undef KVCM_CHAIN_ROWS
+    return launch_status("rmsnorm_chain");
+  }
+  if (f32)
+    rmsnorm_chain_kernel<float><<<R, kChainThreads, 0, s>>>(x, a, a_splits, b, b_splits, static_cast<size_t>(split_stride), wa, wb,
+                                                             combine, w_post, rows, w_pre, static_cast<float*>(out), H, eps, wb_flag);
+  else
+    rmsnorm_chain_kernel<bf16_t><<<R, kChainThreads, 0, s>>>(x, a, a_splits, b, b_splits, static_cast<size_t>(split_stride), wa, wb,
+                                                              combine, w_post, rows, w_pre, static_cast<bf16_t*>(out), H, eps, wb_flag);
   return launch_status("rmsnorm_chain");
 }
 

@@ -63,7 +63,7 @@ def interleaved_steps(lengths, rng):
 def test_chained_norms_against_the_plain_norm():
     from kvcm_amd import ops
     rng = np.random.default_rng(0)
-    for T, H in ((5, 48), (3, 320), (2, 1100)):
+    for T, H in ((5, 48), (3, 320), (2, 1100), (2, 1101), (2, 3000), (3, 5004)):      # rows kept in registers, and rows that are not
         x, a, b = (rng.normal(size=(T, H)) * s for s in (3.0, 0.2, 7.0))
         wa, wb, wp, w = (1.0 + 0.2 * rng.normal(size=H) for _ in range(4))
         eps = 1e-5
