@@ -40,12 +40,23 @@ __global__ void rotary_pairs_table_kernel(const int* __restrict__ positions, flo
   cos_sin[idx] = float2{static_cast<float>(cos(a)), static_cast<float>(sin(a))};
 }
 
+// cos_sin[t, i] = factor * (cos, sin) of position * freqs[i], for rotations whose frequencies are not a plain power
+// law (rescaled for longer contexts pair by pair): the caller brings them as a table, in double precision.
+__global__ void rotary_freq_table_kernel(const int* __restrict__ positions, const double* __restrict__ freqs,
+                                         float2* __restrict__ cos_sin, int T, int half, double factor) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * half) return;
+  const double a = double(positions[idx / half]) * freqs[idx % half];
+  cos_sin[idx] = float2{static_cast<float>(factor * cos(a)), static_cast<float>(factor * sin(a))};
+}
+
 // ------------------------------------------------------- rotation and the page write of a step
 // src [T, nh*d + nkv*d + nkv*dv] 32-bit (q | k | v).  q (rotated) -> q_out [T, nh*d]; k (rotated) and v
-// -> their page slot.  The pair (2i, 2i+1), i < rot/2, is turned; the rest passes.
+// -> their page slot.  halves 0: the pair (2i, 2i+1), i < rot/2, is turned; halves 1: the pair (i, i + rot/2);
+// the rest passes.
 template <class T>
 __global__ void __launch_bounds__(256)
-    rotate_store_kernel(const float* __restrict__ src, int ld, const float2* __restrict__ cos_sin, int rot,
+    rotate_store_kernel(const float* __restrict__ src, int ld, const float2* __restrict__ cos_sin, int rot, int halves,
                         const int* __restrict__ slots, T* __restrict__ q_out, int ldq, T* __restrict__ kcache,
                         T* __restrict__ vcache, int nh, int nkv, int d, int dv, int B) {
   const int row = blockIdx.x;
@@ -55,10 +66,12 @@ __global__ void __launch_bounds__(256)
   for (int e = threadIdx.x; e < (nh + nkv) * d; e += blockDim.x) {
     const int head = e / d, i = e % d;
     float x = r[e];
-    if (i < rot) {      // rot is even: the partner i ^ 1 lies inside the rotated part too
-      const float y = r[size_t(head) * d + (i ^ 1)];
-      const float2 a = cs[i / 2];
-      x = (i & 1) ? __fmaf_rn(x, a.x, __fmul_rn(y, a.y)) : __fmaf_rn(x, a.x, -__fmul_rn(y, a.y));
+    if (i < rot) {      // rot is even: the partner lies inside the rotated part too
+      const int hr = rot / 2;
+      const bool second = halves ? i >= hr : (i & 1);
+      const float y = r[size_t(head) * d + (halves ? (second ? i - hr : i + hr) : (i ^ 1))];
+      const float2 a = cs[halves ? (second ? i - hr : i) : i / 2];
+      x = second ? __fmaf_rn(x, a.x, __fmul_rn(y, a.y)) : __fmaf_rn(x, a.x, -__fmul_rn(y, a.y));
     }
     if (head < nh) store_f(q_out + size_t(row) * ldq + e, x);
     else if (slot >= 0) store_f(kcache + ((size_t(slot / B) * nkv + (head - nh)) * B + slot % B) * d + i, x);
@@ -326,7 +339,17 @@ int kvcm_rotary_pairs_table(const int* positions, float* cos_sin, int T, int dim
   return launch_status("rotary_pairs_table");
 }
 
-int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, const int* slots, void* q_out, int dtype,
+int kvcm_rotary_freq_table(const int* positions, const double* freqs, float* cos_sin, int T, int dims, float factor,
+                           hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && dims > 0 && dims % 2 == 0 && positions && freqs && cos_sin, "rotary_freq_table: bad sizes T=%d dims=%d", T, dims);
+  const int n = T * (dims / 2);
+  rotary_freq_table_kernel<<<(n + 255) / 256, 256, 0, s>>>(positions, freqs, reinterpret_cast<float2*>(cos_sin), T, dims / 2,
+                                                           double(factor));
+  return launch_status("rotary_freq_table");
+}
+
+int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, int halves, const int* slots, void* q_out, int dtype,
                       int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && d > 0 && dv > 0 && B > 0, "rotate_store: bad sizes");
@@ -337,10 +360,10 @@ int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, c
   KVCM_REQUIRE(!slots || (kcache && vcache), "rotate_store: slots without pages");
   const float2* cs = reinterpret_cast<const float2*>(cos_sin);
   if (dtype == kF32)
-    rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, cs, rot, slots, static_cast<float*>(q_out), ldq,
+    rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, cs, rot, halves, slots, static_cast<float*>(q_out), ldq,
                                                   static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, d, dv, B);
   else if (dtype == kBF16)
-    rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, cs, rot, slots, static_cast<bf16_t*>(q_out), ldq,
+    rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, cs, rot, halves, slots, static_cast<bf16_t*>(q_out), ldq,
                                                    static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, d, dv, B);
   else KVCM_REQUIRE(false, "rotate_store: unknown dtype %d", dtype);
   return launch_status("rotate_store");

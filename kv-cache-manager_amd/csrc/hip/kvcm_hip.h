@@ -167,7 +167,9 @@ int kvcm_short_conv_state(const float* in, int ld_in, const float* bias_in, floa
                           hipStream_t s);
 // (attention_window_pool.hip) rotation by interleaved pairs, attention over a window and pooled blocks before it
 int kvcm_rotary_pairs_table(const int* positions, float* cos_sin, int T, int dims, float base, hipStream_t s);
-int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, const int* slots, void* q_out, int dtype,
+int kvcm_rotary_freq_table(const int* positions, const double* freqs, float* cos_sin, int T, int dims, float factor,
+                           hipStream_t s);
+int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, int halves, const int* slots, void* q_out, int dtype,
                       int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B, hipStream_t s);
 int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* pk, float* pv, const int* tables,
                      int table_stride, const int* row_seq, const int* positions, const int* slots, int T, int nkv, int d,
@@ -196,6 +198,28 @@ int kvcm_delta_prepare(const float* k, int ldk, const float* a_lin, int lda, con
 int kvcm_delta_scan(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv, const float* w, const float* au,
                     const float* u, float* o, int ldo, float* state, const int* run_start, const int* seq_start,
                     const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s);
+
+// (stream_norms.hip) a norm without statistics beside the residual additions of a layer whose mixer and feed-forward run
+// side by side; the stream packed with the embedding for a product; a factor on logits; a gate per head; small norms in place
+int kvcm_dyt_norm(float* x, int use_x, const float* a, const float* b, const int* rows, int write_back, const float* w1,
+                  const float* b1, float alpha1, void* out1, const float* w2, const float* b2, float alpha2, void* out2,
+                  int out_dtype, int R, int H, hipStream_t s);
+int kvcm_stream_pack(const float* x, const float* a, const float* b, const float* x0, void* out, int out_dtype, int T, int H,
+                     hipStream_t s);
+int kvcm_scale_rows(float* x, long long n, float factor, hipStream_t s);
+int kvcm_head_gate(void* o, int dtype, int ldo, const float* gate, int ldg, int T, int heads, int dv, hipStream_t s);
+int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const float* w, float eps, int T, hipStream_t s);
+// (mlstm.hip) a matrix memory with exponential gates, walked token by token
+int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* ig, int ldi,
+                    const float* fg, int ldf, const float* i_bias, const float* f_bias, float cap, float q_scale, float* coef,
+                    float* o, int ldo, float* s_state, float* n_state, float* m_state, const int* run_start,
+                    const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s);
+// (moe.hip) a routed feed-forward: the choice of experts, and the experts' two products a row at a time
+int kvcm_moe_route(const float* logits, int ld, int E, int top, int* chosen, float* weight, int T, hipStream_t s);
+int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* chosen, void* act, int T, int K, int F, int top,
+                int E, hipStream_t s);
+int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* chosen, const float* weight, float* out, int T,
+                  int F, int H, int top, int E, hipStream_t s);
 
 // ---- recorded steps ---------------------------------------------------------------------------
 // A step program is the list of launches of one step, recorded once for a step shape and replayed

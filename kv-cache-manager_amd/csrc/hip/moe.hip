@@ -1,0 +1,194 @@
+// A routed feed-forward: every row picks `top` of E small experts by the softmax of its router logits and gets the
+// sum of their outputs weighted by the chosen scores as they are (not renormalized).
+//
+//   moe_route      32-bit router logits [T, E] -> chosen[T, top] (expert numbers, best first; equal scores: the lower
+//                  number) and weight[T, top] (their softmax scores over all E).  One wave per row.
+//   moe_up         act[T, top, F] = a(W_up[e] h) for each row's chosen experts, a = square of relu, rounded to the
+//                  compute dtype
+//   moe_down       out[T, H] (32-bit) = sum over the row's slots of weight * W_down[e] act[slot]
+//
+// The two products here take a row at a time: a workgroup owns one (row, slot) and a stretch of output columns, keeps
+// the row in LDS as 32-bit values and streams the chosen expert's weight rows, a wave per output column, 16 bytes per
+// lane and load, summed across the wave.  A row's result is one fixed sequence of operations on its own data, whatever
+// else the step holds.  Only the chosen experts' weights are read: the kernels of steps with few rows.  Steps with
+// many rows sort their (row, slot) pairs by expert and run tiles on the matrix cores (moe_grouped.hip).
+#include <cfloat>
+
+#include "common.h"
+#include "kvcm_hip.h"
+
+namespace kvcm {
+
+constexpr int kMoeMaxTop = 16;
+
+__global__ void __launch_bounds__(256)
+    moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top, int* __restrict__ chosen,
+                     float* __restrict__ weight, int T) {
+  const int row = blockIdx.x * (256 / kWave) + threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (row >= T) return;
+  const float* z = logits + size_t(row) * ld;
+  float mx = -FLT_MAX;
+  for (int e = lane; e < E; e += kWave) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += kWave) sum += expf(z[e] - mx);
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+  int taken[kMoeMaxTop];
+  for (int s = 0; s < top; ++s) {
+    float best = -FLT_MAX;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += kWave) {
+      bool used = false;
+      for (int p = 0; p < s; ++p) used |= taken[p] == e;
+      const float val = z[e];
+      if (!used && (val > best || (val == best && e < at))) { best = val; at = e; }
+    }
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, kWave);
+      const int oa = __shfl_xor(at, o, kWave);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    taken[s] = at;
+    if (lane == 0) {
+      chosen[size_t(row) * top + s] = at;
+      weight[size_t(row) * top + s] = expf(best - mx) * inv;
+    }
+  }
+}
+
+template <class T> struct Piece;
+template <> struct Piece<float> { static constexpr int N = 4; };
+template <> struct Piece<bf16_t> { static constexpr int N = 8; };
+
+__device__ __forceinline__ void unpack16(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+__device__ __forceinline__ void unpack16(const bf16_t* p, float* f) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  f[0] = bf16_bits_to_float(v.x & 0xffffu); f[1] = bf16_bits_to_float(v.x >> 16);
+  f[2] = bf16_bits_to_float(v.y & 0xffffu); f[3] = bf16_bits_to_float(v.y >> 16);
+  f[4] = bf16_bits_to_float(v.z & 0xffffu); f[5] = bf16_bits_to_float(v.z >> 16);
+  f[6] = bf16_bits_to_float(v.w & 0xffffu); f[7] = bf16_bits_to_float(v.w >> 16);
+}
+
+// sum over k of xs[k] * w[k], w a stored row of K values, xs the row in LDS; the wave's lanes take pieces in turn
+template <class T>
+__device__ __forceinline__ float wave_dot(const float* xs, const T* w, int K, int lane, bool vec) {
+  constexpr int N = Piece<T>::N;
+  float acc = 0.f;
+  if (vec) {
+    for (int k = lane * N; k < K; k += kWave * N) {
+      float f[N];
+      unpack16(w + k, f);
+#pragma unroll
+      for (int e = 0; e < N; ++e) acc = fmaf(xs[k + e], f[e], acc);
+    }
+  } else {
+    for (int k = lane; k < K; k += kWave) acc = fmaf(xs[k], load_f(w + k), acc);
+  }
+  return wave_sum(acc);
+}
+
+constexpr int kMoeCols = 32;      // output columns of a workgroup (8 a wave)
+
+// grid (T * top, column blocks).  h [T, K] in T; w_up [E, F, K]; act [T * top, F].
+template <class T>
+__global__ void __launch_bounds__(256)
+    moe_up_kernel(const T* __restrict__ h, int ldh, const T* __restrict__ w_up, const int* __restrict__ chosen,
+                  T* __restrict__ act, int K, int F, int top, int E) {
+  extern __shared__ float xs[];
+  const int item = blockIdx.x, row = item / top;
+  const int e = chosen[item];
+  for (int k = threadIdx.x; k < K; k += 256) xs[k] = load_f(h + size_t(row) * ldh + k);
+  __syncthreads();
+  if (e < 0 || e >= E) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const bool vec = K % Piece<T>::N == 0;
+  const T* w = w_up + size_t(e) * F * K;
+  for (int c = blockIdx.y * kMoeCols + wave; c < min(F, (blockIdx.y + 1) * kMoeCols); c += 256 / kWave) {
+    const float z = wave_dot(xs, w + size_t(c) * K, K, lane, vec);
+    const float r = fmaxf(z, 0.f);
+    if (lane == 0) store_f(act + size_t(item) * F + c, r * r);
+  }
+}
+
+// grid (T, column blocks).  act [T * top, F] in T; w_down [E, H, F]; out [T, H] 32-bit.
+template <class T>
+__global__ void __launch_bounds__(256)
+    moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down, const int* __restrict__ chosen,
+                    const float* __restrict__ weight, float* __restrict__ out, int F, int H, int top, int E) {
+  extern __shared__ float xs[];      // [top][F]
+  const int row = blockIdx.x;
+  for (int k = threadIdx.x; k < top * F; k += 256) xs[k] = load_f(act + size_t(row) * top * F + k);
+  __syncthreads();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const bool vec = F % Piece<T>::N == 0;
+  for (int c = blockIdx.y * kMoeCols + wave; c < min(H, (blockIdx.y + 1) * kMoeCols); c += 256 / kWave) {
+    float acc = 0.f;
+    for (int s = 0; s < top; ++s) {
+      const int e = chosen[size_t(row) * top + s];
+      if (e < 0 || e >= E) continue;
+      const float z = wave_dot(xs + s * F, w_down + (size_t(e) * H + c) * F, F, lane, vec);
+      acc = fmaf(weight[size_t(row) * top + s], z, acc);
+    }
+    if (lane == 0) out[size_t(row) * H + c] = acc;
+  }
+}
+
+}  // namespace kvcm
+
+using namespace kvcm;
+
+extern "C" {
+
+int kvcm_moe_route(const float* logits, int ld, int E, int top, int* chosen, float* weight, int T, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E && ld >= E, "moe_route: bad sizes T=%d experts=%d top=%d", T, E, top);
+  KVCM_REQUIRE(top <= kMoeMaxTop, "moe_route: %d experts a row are not supported (up to %d)", top, kMoeMaxTop);
+  moe_route_kernel<<<(T + 3) / 4, 256, 0, s>>>(logits, ld, E, top, chosen, weight, T);
+  return launch_status("moe_route");
+}
+
+// h [T, K] and act [T * top, F] in dtype; w_up [E, F, K] contiguous.  act = square(relu(W_up[chosen] h)).
+int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* chosen, void* act, int T, int K, int F, int top,
+                int E, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && K > 0 && F > 0 && top > 0 && E > 0 && ldh >= K, "moe_up: bad sizes");
+  KVCM_REQUIRE(static_cast<long long>(T) * top < (1ll << 31) && (F + kMoeCols - 1) / kMoeCols <= 65535, "moe_up: too many rows or columns");
+  KVCM_REQUIRE(K * sizeof(float) <= 64 * 1024, "moe_up: rows of %d values do not fit the local memory", K);
+  KVCM_REQUIRE(reinterpret_cast<uintptr_t>(w_up) % 16 == 0, "moe_up: weights must be 16-byte aligned");
+  const dim3 grid(T * top, (F + kMoeCols - 1) / kMoeCols);
+  if (dtype == kF32)
+    moe_up_kernel<float><<<grid, 256, K * sizeof(float), s>>>(static_cast<const float*>(h), ldh, static_cast<const float*>(w_up),
+                                                             chosen, static_cast<float*>(act), K, F, top, E);
+  else if (dtype == kBF16)
+    moe_up_kernel<bf16_t><<<grid, 256, K * sizeof(float), s>>>(static_cast<const bf16_t*>(h), ldh, static_cast<const bf16_t*>(w_up),
+                                                              chosen, static_cast<bf16_t*>(act), K, F, top, E);
+  else KVCM_REQUIRE(false, "moe_up: unknown dtype %d", dtype);
+  return launch_status("moe_up");
+}
+
+// act [T * top, F] in dtype; w_down [E, H, F] contiguous; out [T, H] 32-bit.
+int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* chosen, const float* weight, float* out, int T,
+                  int F, int H, int top, int E, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && H > 0 && F > 0 && top > 0 && E > 0, "moe_down: bad sizes");
+  KVCM_REQUIRE(static_cast<size_t>(top) * F * sizeof(float) <= 64 * 1024, "moe_down: %d activations of %d values do not fit the local memory", top, F);
+  KVCM_REQUIRE(reinterpret_cast<uintptr_t>(w_down) % 16 == 0, "moe_down: weights must be 16-byte aligned");
+  KVCM_REQUIRE((H + kMoeCols - 1) / kMoeCols <= 65535, "moe_down: too many columns");
+  const dim3 grid(T, (H + kMoeCols - 1) / kMoeCols);
+  const size_t lds = static_cast<size_t>(top) * F * sizeof(float);
+  if (dtype == kF32)
+    moe_down_kernel<float><<<grid, 256, lds, s>>>(static_cast<const float*>(act), static_cast<const float*>(w_down), chosen, weight,
+                                                 out, F, H, top, E);
+  else if (dtype == kBF16)
+    moe_down_kernel<bf16_t><<<grid, 256, lds, s>>>(static_cast<const bf16_t*>(act), static_cast<const bf16_t*>(w_down), chosen,
+                                                  weight, out, F, H, top, E);
+  else KVCM_REQUIRE(false, "moe_down: unknown dtype %d", dtype);
+  return launch_status("moe_down");
+}
+
+}  // extern "C"

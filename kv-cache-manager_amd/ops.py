@@ -94,7 +94,17 @@ def _declare(lib):
     fn("kvcm_short_conv", vp, i, vp, vp, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_short_conv_state", vp, i, vp, vp, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_rotary_pairs_table", vp, vp, i, i, f, vp)
-    fn("kvcm_rotate_store", vp, i, vp, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_rotate_store", vp, i, vp, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_rotary_freq_table", vp, vp, vp, i, i, f, vp)
+    fn("kvcm_dyt_norm", vp, i, vp, vp, vp, i, vp, vp, f, vp, vp, vp, f, vp, i, i, i, vp)
+    fn("kvcm_stream_pack", vp, vp, vp, vp, vp, i, i, i, vp)
+    fn("kvcm_scale_rows", vp, C.c_longlong, f, vp)
+    fn("kvcm_head_gate", vp, i, i, vp, i, i, i, i, vp)
+    fn("kvcm_rms_groups", vp, i, i, i, i, vp, f, i, vp)
+    fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_moe_route", vp, i, i, i, vp, vp, i, vp)
+    fn("kvcm_moe_up", vp, i, i, vp, vp, vp, i, i, i, i, i, vp)
+    fn("kvcm_moe_down", vp, i, vp, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_pool_update", vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp)
     fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
@@ -1075,10 +1085,10 @@ def rotary_pairs_table(positions, out, dims, base, rows=None):
     return out
 
 
-def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kcache=None, vcache=None, rows=None):
+def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kcache=None, vcache=None, rows=None, halves=False):
     """qkv: 32-bit rows [q (nh*d) | k (nkv*d) | v (nkv*dv)].  The first ``rot`` entries of every q and k head are
-    turned by interleaved pairs with the table ``cos_sin``; q goes to q_out [T, nh*d], k and v to their page slots
-    (keys [pages, nkv, B, d], values [pages, nkv, dv, B])."""
+    turned with the table ``cos_sin``, by interleaved pairs (2i, 2i+1) or, with ``halves``, by pairs (i, i + rot/2);
+    q goes to q_out [T, nh*d], k and v to their page slots (keys [pages, nkv, B, d], values [pages, nkv, dv, B])."""
     T = q_out.shape[0] if rows is None else rows
     _f32rows(qkv, "qkv", (nh + nkv) * d + nkv * dv)
     _rows2d(q_out, "q_out")
@@ -1094,7 +1104,7 @@ def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kc
     if rot:
         _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.numel() >= T * rot,
               "cos_sin must be float32 [rows, rot/2, 2]")
-    _call("kvcm_rotate_store", _ptr(qkv), qkv.stride(0), _ptr(cos_sin), rot, _ptr(slots), _ptr(q_out), _DT[q_out.dtype],
+    _call("kvcm_rotate_store", _ptr(qkv), qkv.stride(0), _ptr(cos_sin), rot, 1 if halves else 0, _ptr(slots), _ptr(q_out), _DT[q_out.dtype],
           q_out.stride(0), _ptr(kcache), _ptr(vcache), T, nh, nkv, d, dv, B, _stream())
 
 
@@ -1241,3 +1251,148 @@ def delta_scan(r, k, v, w, au, u, o, state, step, heads, dk, dv):
           _ptr(o), o.stride(0), _ptr(state), _ptr(step.run_start), _ptr(step.seq_start), _ptr(step.state_slots), step.seqs,
           heads, dk, dv, _stream())
     return o
+
+
+# ------------------------------------------- a stream whose layers run mixer and feed-forward side by side
+def rotary_freq_table(positions, freqs, out, dims, factor=1.0, rows=None):
+    """out[t, i] = factor * (cos, sin) of positions[t] * freqs[i], float32 [rows, dims/2, 2]; freqs: float64 [dims/2] on
+    the GPU (frequencies that are no plain power law: rescaled pair by pair for longer contexts)."""
+    T = out.shape[0] if rows is None else rows
+    _i32(positions, "positions", T)
+    _need(freqs.dtype == torch.float64 and freqs.is_contiguous() and freqs.is_cuda and freqs.numel() == dims // 2,
+          "freqs must be float64 [dims/2] on the GPU")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.is_cuda and out.numel() >= T * dims,
+          "the table must be float32 [rows, dims/2, 2]")
+    _call("kvcm_rotary_freq_table", _ptr(positions), _ptr(freqs), _ptr(out), T, dims, float(factor), _stream())
+    return out
+
+
+class DytNorm:
+    """One norm tanh(alpha x) * weight + bias as ``dyt_norm`` takes it: (weight, bias: float32 [H]; alpha: a number)."""
+
+    def __init__(self, weight, bias, alpha):
+        self.weight, self.bias, self.alpha = weight, bias, float(alpha)
+
+
+def dyt_norm(x, first=None, out1=None, second=None, out2=None, add_a=None, add_b=None, rows=None, replace=False):
+    """x += add_a + add_b (``replace``: x = add_a + add_b), written back unless ``rows`` gathers; then
+    out1 = first(x), out2 = second(x), each tanh(alpha x) * weight + bias rounded once to the output's dtype.
+    x, add_a, add_b: float32 [T, H]; out1, out2 [R, H]; rows: int32 [R] source rows (None: row r)."""
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.is_cuda and x.dim() == 2, "x must be contiguous float32 [T, H]")
+    T, H = x.shape
+    for t, n in ((add_a, "add_a"), (add_b, "add_b")):
+        if t is not None:
+            _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and tuple(t.shape) == (T, H), f"{n} must match x")
+    _need(add_a is not None or add_b is None, "dyt_norm: a second addition needs a first")
+    _need(not replace or add_a is not None, "dyt_norm: nothing to replace x with")
+    R, dt = T, 0
+    for norm, out in ((first, out1), (second, out2)):
+        _need((norm is None) == (out is None), "dyt_norm: every output needs its norm")
+        if out is not None:
+            _need(out.is_cuda and out.is_contiguous() and out.dim() == 2 and out.shape[1] == H, "out must be contiguous [R, H]")
+            _f32(norm.weight, "the norm weight", H)
+            _f32(norm.bias, "the norm bias", H)
+            R, dt = out.shape[0], _DT[out.dtype]
+    if out1 is not None and out2 is not None:
+        _need(out1.shape == out2.shape and out1.dtype == out2.dtype, "dyt_norm: the two outputs must agree")
+    if rows is not None:
+        _i32(rows, "rows", R)
+    else:
+        _need(R <= T, "x has fewer rows than the output")
+    write_back = 1 if (rows is None and add_a is not None) else 0
+    _need(write_back or out1 is not None or out2 is not None, "dyt_norm: nothing to do")
+    _call("kvcm_dyt_norm", _ptr(x), 0 if replace else 1, _ptr(add_a), _ptr(add_b), _ptr(rows), write_back,
+          _ptr(first.weight) if first else 0, _ptr(first.bias) if first else 0, first.alpha if first else 0.0, _ptr(out1),
+          _ptr(second.weight) if second else 0, _ptr(second.bias) if second else 0, second.alpha if second else 0.0, _ptr(out2),
+          dt, R, H, _stream())
+
+
+def stream_pack(x, x0, out, add_a=None, add_b=None):
+    """out[T, 2H] = [x + add_a + add_b | x0] in out's dtype; x, x0 and the additions float32 [T, H]."""
+    T, H = x.shape
+    for t, n in ((x, "x"), (x0, "x0"), (add_a, "add_a"), (add_b, "add_b")):
+        if t is not None:
+            _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and tuple(t.shape) == (T, H), f"{n} must be float32 [T, H]")
+    _need(add_a is not None or add_b is None, "stream_pack: a second addition needs a first")
+    _need(out.is_cuda and out.is_contiguous() and tuple(out.shape) == (T, 2 * H), "out must be contiguous [T, 2H]")
+    _call("kvcm_stream_pack", _ptr(x), _ptr(add_a), _ptr(add_b), _ptr(x0), _ptr(out), _DT[out.dtype], T, H, _stream())
+    return out
+
+
+def scale_rows(x, factor):
+    """x *= factor in place (float32)."""
+    _f32(x, "x")
+    _call("kvcm_scale_rows", _ptr(x), x.numel(), float(factor), _stream())
+    return x
+
+
+def head_gate(o, gate, heads, dv, rows=None):
+    """o[r, h, :] *= sigmoid(gate[r, h]) in place; o [T, >= heads*dv] in the compute dtype, gate float32 rows of >= heads."""
+    T = o.shape[0] if rows is None else rows
+    _rows2d(o, "o")
+    _f32rows(gate, "gate", heads)
+    _need(o.is_cuda and o.shape[1] >= heads * dv and gate.shape[0] >= T and o.shape[0] >= T, "head_gate: shapes do not agree")
+    _call("kvcm_head_gate", _ptr(o), _DT[o.dtype], o.stride(0), _ptr(gate), gate.stride(0), T, heads, dv, _stream())
+    return o
+
+
+def rms_groups(x, col0, size, groups, weight, eps, rows=None):
+    """In place on float32 rows: each of ``groups`` stretches of ``size`` columns from col0 on is divided by its root mean
+    square (eps inside the root) and multiplied by weight[0 .. size)."""
+    T = x.shape[0] if rows is None else rows
+    _f32rows(x, "x", col0 + size * groups)
+    _f32(weight, "weight", size)
+    _call("kvcm_rms_groups", _ptr(x), x.stride(0), col0, size, groups, _ptr(weight), float(eps), T, _stream())
+    return x
+
+
+def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, coef, o, s_state, n_state, m_state, step, heads, dk, dv):
+    """The matrix memory with exponential gates over the step's runs (csrc/hip/mlstm.hip).  q, k [T, heads*dk], v [T, heads*dv],
+    gate_in, gate_keep [T, heads] (projections without biases): 32-bit rows; coef: float32 scratch of 4 T heads values;
+    states [slots, heads, dk, dv], [slots, heads, dk], [slots, heads]."""
+    T = o.shape[0]
+    for t, n, c in ((q, "q", heads * dk), (k, "k", heads * dk), (v, "v", heads * dv), (o, "o", heads * dv), (gate_in, "gate_in", heads),
+                    (gate_keep, "gate_keep", heads)):
+        _f32rows(t, n, c)
+        _need(t.shape[0] >= T, f"{n} has too few rows")
+    _f32(in_bias, "in_bias", heads)
+    _f32(keep_bias, "keep_bias", heads)
+    _f32(coef, "coef", 4 * T * heads)
+    for t, n, shape in ((s_state, "s_state", (heads, dk, dv)), (n_state, "n_state", (heads, dk)), (m_state, "m_state", (heads,))):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and tuple(t.shape[1:]) == shape, f"{n} must be float32 [slots, {shape}]")
+    _call("kvcm_mlstm_scan", _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(gate_in), gate_in.stride(0),
+          _ptr(gate_keep), gate_keep.stride(0), _ptr(in_bias), _ptr(keep_bias), float(cap), float(q_scale), _ptr(coef), _ptr(o),
+          o.stride(0), _ptr(s_state), _ptr(n_state), _ptr(m_state), _ptr(step.run_start), _ptr(step.seq_start),
+          _ptr(step.state_slots), step.seqs, heads, dk, dv, _stream())
+    return o
+
+
+def moe_route(logits, experts, top, chosen, weight, rows=None):
+    """chosen[T, top] (int32) and weight[T, top] (float32): the ``top`` experts with the largest softmax scores over all
+    ``experts`` of each row's 32-bit router logits, best first, with those scores."""
+    T = chosen.shape[0] if rows is None else rows
+    _f32rows(logits, "logits", experts)
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.is_cuda and chosen.shape[1] == top and chosen.shape[0] >= T,
+          "chosen must be int32 [T, top]")
+    _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.is_cuda and tuple(weight.shape) == tuple(chosen.shape),
+          "weight must be float32 [T, top]")
+    _call("kvcm_moe_route", _ptr(logits), logits.stride(0), experts, top, _ptr(chosen), _ptr(weight), T, _stream())
+
+
+def moe_rows(h, w_up, w_down, chosen, weight, act, out):
+    """out[T, H] (float32) = sum over a row's chosen experts e of weight * W_down[e] square(relu(W_up[e] h)), a row at a
+    time, reading only the chosen experts.  h [T, K]; w_up [E, F, K]; w_down [E, H, F]; act: work memory [T * top, F]."""
+    T, K = h.shape
+    E, F, _ = w_up.shape
+    H, top = w_down.shape[1], chosen.shape[1]
+    _rows2d(h, "h")
+    _need(h.is_cuda and h.dtype == w_up.dtype == w_down.dtype == act.dtype, "moe_rows: operands must share one dtype")
+    _need(w_up.is_contiguous() and w_down.is_contiguous() and tuple(w_up.shape) == (E, F, K) and tuple(w_down.shape) == (E, H, F),
+          "moe_rows: expert weights must be [E, F, K] and [E, H, F]")
+    _need(act.is_contiguous() and act.shape[0] >= T * top and act.shape[1] == F, "act must be [T * top, F]")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H), "out must be float32 [T, H]")
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.shape[0] >= T, "chosen must be int32 [T, top]")
+    _need(weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == tuple(chosen.shape), "weight must match chosen")
+    _call("kvcm_moe_up", _ptr(h), _DT[h.dtype], h.stride(0), _ptr(w_up), _ptr(chosen), _ptr(act), T, K, F, top, E, _stream())
+    _call("kvcm_moe_down", _ptr(act), _DT[act.dtype], _ptr(w_down), _ptr(chosen), _ptr(weight), _ptr(out), T, F, H, top, E, _stream())
+    return out

@@ -49,6 +49,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     max_position: int = 0
+    keep_embedding: bool = False      # the embedding's output stays at hand for the layers (step.shared["embedding_output"])
 
 
 # ---------------------------------------------------------------------------------- weights
@@ -66,6 +67,8 @@ class ParamSpec:
     @property
     def shape(self):
         first = self.sources[0][1]
+        if not first:
+            return ()      # a scalar
         return (sum(s[1][0] for s in self.sources),) + tuple(first[1:])
 
 

@@ -243,7 +243,8 @@ class TokenEmbedding(Embedding):
 @HEADS.register("linear_head")
 class LinearHead(Head):
     """logits = h @ table^T in 32-bit, only for the rows that are asked for
-    (src/model/llama.cpp:126-128).  params: vocab_size, tied (use the embedding's table)."""
+    (src/model/llama.cpp:126-128).  params: vocab_size, tied (use the embedding's table), scale (a factor on the
+    logits, default 1: applied to the 32-bit logits)."""
 
     capturable = True
 
@@ -261,6 +262,8 @@ class LinearHead(Head):
 
     def forward(self, step, h, out):
         self.ctx.ops.gemm(h, self.w["table"], out, tuning=step.tune_products)
+        if float(self.params.get("scale", 1.0)) != 1.0:
+            self.ctx.ops.scale_rows(out, self.params["scale"])
         return out
 
 

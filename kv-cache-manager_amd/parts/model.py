@@ -6,12 +6,12 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, Registry
+from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, STREAM_PARTS, Registry
 from .base import BuildContext, KVCacheNeed, ModelSpec, Part, StateNeed, as_tensor
 
 # registries by the names a block arrangement may use in ``part_registries``
 _REGISTRY_NAMES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "ffn": FEED_FORWARDS, "norm": NORMS,
-                   "position": POSITIONS}
+                   "position": POSITIONS, "stream": STREAM_PARTS}
 
 
 def _registry_for(slot, block_class=None):
@@ -227,6 +227,11 @@ class Model:
         the last block's output that is not added to it yet."""
         x = step.ws("residual", (step.rows, self.spec.hidden_size), torch.float32)
         self.embedding.forward(step, x)
+        if self.spec.keep_embedding:
+            # a copy of the embedding's output for parts that mix it into the stream again later (step.shared)
+            x0 = step.ws("embedding_output", (step.rows, self.spec.hidden_size), torch.float32)
+            self.embedding.forward(step, x0)
+            step.shared["embedding_output"] = x0
         pending = None
         for i in self.spec.schedule:
             pending = self.blocks[i].forward(step, x, pending)

@@ -131,3 +131,57 @@ class GeneralDeltaMixer(_StatefulMixer):
         gated = step.ws("delta_gated", (T, D))
         ops.head_norm_gate(o, g, w["norm"], gated, heads, d, p["eps"])
         return linear32(self.ctx, step, gated, w["w_o"], "delta_out")
+
+
+@MIXERS.register("matrix_memory")
+class MatrixMemoryMixer(_StatefulMixer):
+    """A matrix memory with exponential gates (the mLSTM cell).  q, k, v, the output gate g and one input and one forget
+    gate per head are one fused product; q is scaled by dim^(-1/2); li = cap tanh((W_i h + b_i) / cap),
+    lf = logsigmoid(cap tanh((W_f h + b_f) / cap)); m' = max(lf + m, li), S' = exp(lf + m - m') S + exp(li - m') k v^T, n'
+    likewise with k alone, o = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6); every head's o is divided by its root mean
+    square, times a weight over all heads, times sigmoid(g), then the output projection.  S, n and m start at 0.
+    params: heads, dim, vdim, gate_cap, eps.  Tensors under the prefix: q, k, v, g, i, i.b, f, f.b, norm, o.
+    Keeps S [heads, dim, vdim], n [heads, dim] and m [heads] per request, 32-bit."""
+
+    def param_specs(self):
+        H, p, pre = self.ctx.hidden_size, self.params, self.prefix
+        heads, d, dv = p["heads"], p["dim"], p["vdim"]
+        sizes = (("q", heads * d), ("k", heads * d), ("v", heads * dv), ("g", heads * dv), ("i", heads), ("f", heads))
+        return [ParamSpec("w_proj", tuple((pre + n, (c, H)) for n, c in sizes)),
+                ParamSpec("in_bias", ((pre + "i.b", (heads,)),), role="vector"),
+                ParamSpec("keep_bias", ((pre + "f.b", (heads,)),), role="vector"),
+                ParamSpec("norm", ((pre + "norm", (heads * dv,)),), role="vector"),
+                ParamSpec("w_o", ((pre + "o", (H, heads * dv)),))]
+
+    def bind(self, tensors):
+        w = tensors["w_proj"]
+        extra = -w.shape[0] % 16      # the few-row products take widths that are multiples of 16
+        if extra:
+            w = torch.cat([w, torch.zeros(extra, w.shape[1], dtype=w.dtype, device=w.device)], 0)
+        small = f32_params({k: tensors[k] for k in ("in_bias", "keep_bias", "norm")})
+        Mixer.bind(self, {**tensors, **small, "w_proj": w})
+
+    def cache_needs(self):
+        p = self.params
+        return {"memory": StateNeed((p["heads"], p["dim"], p["vdim"]), torch.float32),
+                "normalizer": StateNeed((p["heads"], p["dim"]), torch.float32),
+                "maximum": StateNeed((p["heads"],), torch.float32)}
+
+    def flops(self, rows, attended=0):
+        p = self.params
+        return super().flops(rows) + rows * p["heads"] * (4.0 * p["dim"] * p["vdim"] + 4.0 * p["dim"])
+
+    def forward(self, step, h):
+        ops, p, w = self.ctx.ops, self.params, self.w
+        heads, d, dv = p["heads"], p["dim"], p["vdim"]
+        T = step.rows
+        proj = linear32(self.ctx, step, h, w["w_proj"], "memory_proj")
+        at = [0, heads * d, 2 * heads * d, 2 * heads * d + heads * dv, 2 * heads * (d + dv), 2 * heads * (d + dv) + heads]
+        q, k, v, g, gi, gf = (proj[:, lo:] for lo in at)
+        coef = step.ws("memory_factors", (T, 4 * heads), torch.float32)
+        o = step.ws("memory_o", (T, heads * dv), torch.float32)
+        ops.mlstm_scan(q, k, v, gi, gf, w["in_bias"], w["keep_bias"], p["gate_cap"], float(d) ** -0.5, coef, o,
+                       self.state("memory"), self.state("normalizer"), self.state("maximum"), step, heads, d, dv)
+        gated = step.ws("memory_gated", (T, heads * dv))
+        ops.head_norm_gate(o, g, w["norm"], gated, heads, dv, p["eps"])
+        return linear32(self.ctx, step, gated, w["w_o"], "memory_out")

@@ -54,4 +54,5 @@ POSITIONS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("output head")
+STREAM_PARTS = Registry("stream part")      # parts that act on the residual stream itself, between layers
 ARCHITECTURES = Registry("architecture")

@@ -118,6 +118,7 @@ def load_weights(model, source, compute_dtype: torch.dtype, device) -> int:
     """Checks, then binds every part's tensors on ``device``.  Returns the bytes now on the device."""
     check_against(model, source)
     total = 0
+    loaded = {}      # (sources, dtype) -> tensor: parts that name the same tensors (layers that run again with caches of their own) share them
     for part in model.every_part():
         bound = {}
         for spec in part.param_specs():
@@ -125,7 +126,16 @@ def load_weights(model, source, compute_dtype: torch.dtype, device) -> int:
             if len(dtypes) != 1:
                 raise WeightsError(f"{spec.sources[0][0]} and the tensors fused with it are stored in different precisions")
             dt = dtypes.pop()
+            key = (tuple(n for n, _ in spec.sources), dt)
+            if key in loaded:
+                bound[spec.name] = loaded[key]
+                continue
             shapes = [tuple(source.shape(name)) for name, _ in spec.sources]      # the stored ones: a declared -1 is open
+            if shapes == [()]:      # a stored scalar
+                out = source.get(spec.sources[0][0]).to(device=device, dtype=dt).reshape(())
+                bound[spec.name] = loaded[key] = out
+                total += out.element_size()
+                continue
             if len({sh[1:] for sh in shapes}) != 1:
                 raise WeightsError(f"{spec.sources[0][0]} and the tensors fused with it do not have the same row length")
             out = torch.empty((sum(sh[0] for sh in shapes),) + shapes[0][1:], dtype=dt, device=device)
@@ -133,7 +143,7 @@ def load_weights(model, source, compute_dtype: torch.dtype, device) -> int:
             for (name, _), shape in zip(spec.sources, shapes):
                 out[row:row + shape[0]].copy_(source.get(name).to(dt))
                 row += shape[0]
-            bound[spec.name] = out
+            bound[spec.name] = loaded[key] = out
             total += out.numel() * out.element_size()
         part.bind(bound)
     model.finish_binding()
