@@ -257,7 +257,8 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
       if (wide_v) {
         // all of the chunk's pieces (N tokens of one page each) are requested at once, from places clamped into the
         // context; probabilities of tokens before the window are zero, values beyond the context are cut
-        const int last_piece = ((ctx - 1) / N) * N;
+        // (pages that the window has passed may have been given back: nothing before the window's first piece is read)
+        const int last_piece = ((ctx - 1) / N) * N, first_piece = (first / N) * N;
 #pragma unroll
         for (int i = 0; i < COLS; ++i) {
           if (i * kWave >= dv) break;      // the same for every lane: 64 columns at a time, each with its own trip of loads
@@ -266,7 +267,8 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
           float f[kWave / N][N];
 #pragma unroll
           for (int g = 0; g < kWave / N; ++g) {
-            const int tj = c0 + g * N < last_piece ? c0 + g * N : last_piece;
+            const int tg = c0 + g * N < first_piece ? first_piece : c0 + g * N;
+            const int tj = tg < last_piece ? tg : last_piece;
             unpack_piece(vcache + size_t(table[tj / B]) * vpage + kvh * vhead + size_t(col) * B + tj % B, f[g]);
           }
           float acc = o[i];
@@ -275,7 +277,7 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
 #pragma unroll
             for (int e = 0; e < N; ++e) {
               const int j = g * N + e;
-              acc = fmaf(ps[j], j < j_hi ? f[g][e] : 0.f, acc);
+              acc = fmaf(ps[j], (j >= j_lo && j < j_hi) ? f[g][e] : 0.f, acc);
             }
           if (cc < dv) o[i] = acc;
         }

@@ -95,7 +95,9 @@ __global__ void __launch_bounds__(256)
     for (int qq = 0; qq < KQ; ++qq) {
       const int e = tid + qq * 256;
       const int key = (e / (DP / 8)) % kChunk, k = (e % (DP / 8)) * 8, t = c0 + key;
-      const int tc = t <= p_last ? t : p_last, kc = k < d ? k : d - 8;
+      // (pages that the window has passed may have been given back: nothing before the tile's first seen token is read)
+      const int tl = t < t_lo ? t_lo : t;
+      const int tc = tl <= p_last ? tl : p_last, kc = k < d ? k : d - 8;
       const uint4 v = *reinterpret_cast<const uint4*>(kcache + ((size_t(table[tc / B]) * nkv + kvh) * B + tc % B) * d + kc);
       kreg[qq] = (t <= p_last && k < d) ? v : uint4{0u, 0u, 0u, 0u};
     }
@@ -103,7 +105,8 @@ __global__ void __launch_bounds__(256)
     for (int qq = 0; qq < VQ; ++qq) {
       const int e = tid + qq * 256;
       const int cc = (e / (kChunk / 8)) % DVP, piece = e % (kChunk / 8), t = c0 + piece * 8;
-      const int tc = t <= p_last ? t : (p_last / 8) * 8, ccl = cc < dv ? cc : dv - 1;
+      const int tl = t < (t_lo / 8) * 8 ? (t_lo / 8) * 8 : t;
+      const int tc = tl <= p_last ? tl : (p_last / 8) * 8, ccl = cc < dv ? cc : dv - 1;
       uint4 v = *reinterpret_cast<const uint4*>(vcache + ((size_t(table[tc / B]) * nkv + kvh) * dv + ccl) * B + tc % B);
       v = keep_first_bf16(v, p_last + 1 - t < 8 ? p_last + 1 - t : 8);      // beyond the newest token: whatever was there
       vreg[qq] = cc < dv ? v : uint4{0u, 0u, 0u, 0u};
