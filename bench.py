@@ -3,7 +3,7 @@
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512] [--layers L]
                   [--sizes tinyllama-1.1b|llama-2-7b|llama-3-8b] [--context-limit 2048] [--prefill-tokens 2048]
                   [--tune-products off|heuristic|all] [--no-points] [--only-prefill]
-  python bench.py --design kasuvik [--design-sizes 2048,4096] [--layers 4] [--prefill-tokens 2048] [--steps K]
+  python bench.py --design kasuvik|furapel [--design-sizes 2048,4096] [--layers 4] [--prefill-tokens 2048] [--steps K]
 
 A "step" is one decode step of the whole engine (schedule, batch metadata, upload, model step on
 the GPU, sampling, download, update).  W untimed steps, then exactly K timed steps between two
@@ -14,6 +14,10 @@ the same at batch 1 and 64, a 2,048-token prefill, and the decode step's memory 
 Kasuvik decoder (attention over a window and pooled blocks beside a selective scan, and delta-rule layers) at
 layer sizes that resemble served models, beside the Llama decoder at equal width, heads, feed-forward and
 depth, both with random weights through the same engine.  One JSON line with both designs' figures per size.
+
+--design furapel does the same for the Furapel decoder (side-by-side layers with dynamic tanh norms: gated grouped-query
+attention, latent attention over a window, a matrix memory with exponential gates, routed experts) beside the Kasuvik
+and the Llama decoder at equal width, heads, active feed-forward width and depth.
 """
 import argparse
 import json
@@ -162,6 +166,29 @@ def kasuvik_pair(width, layers, vocab=32000):
     return kas, llama
 
 
+# Furapel at a width: (latent size, window of the latent attention, experts, experts a row); the other sizes are DESIGN_SIZES'
+FURAPEL_SIZES = {2048: (128, 512, 8, 2), 4096: (128, 1024, 8, 2)}
+
+
+def furapel_config(width, layers, vocab=32000):
+    """A Furapel configuration at a width of DESIGN_SIZES: layers latent attention, gated attention, matrix memory, gated
+    attention in turn, each beside ``experts`` experts of which a row uses ``top`` (together as wide as the dense
+    feed-forward of the same width), the first layer led in by the product that mixes the embedding in again."""
+    from kvcm_amd.config.furapel_config import FurapelConfig
+    nh, nkv, hd, ff = DESIGN_SIZES[width][:4]
+    rank, window, experts, top = FURAPEL_SIZES[width]
+    mlp = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": experts, "top": top}}
+    attention = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                 "rot": {"dims": hd // 2, "base": 10000.0, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    latent = {"heads": nh, "dim": hd, "vdim": hd, "kv_rank": rank, "scale": hd ** -0.5, "mask": {"size": window}}
+    memory = {"heads": nh, "dim": hd, "vdim": hd, "gate_cap": 15.0}
+    kinds = [("latent_attention", latent), ("attention", attention), ("mlstm", memory), ("attention", attention)]
+    listed = [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": mlp} for i in range(layers)]
+    return FurapelConfig.from_dict({"architecture": "Furapel", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+                                    "norm": {"eps": 1e-6}, "logit_scale": 1.0, "layers": listed,
+                                    "loop": {"start": 0, "stop": 1, "times": 1}})
+
+
 def design_main(args):
     import torch
     from kvcm_amd.config.engine_config import EngineConfig
@@ -173,15 +200,20 @@ def design_main(args):
     limit = max(2048, -(-(T + 64) // 64) * 64, -(-(args.prompt_len + steps + warmup + 64) // 64) * 64)
     dt = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
-    record = {"metric": "prefill and decode tok/s of the Kasuvik decoder beside the Llama decoder at equal sizes", "dtype": key,
+    first = args.design
+    record = {"metric": "prefill and decode tok/s of the %s decoder beside the %s at equal sizes"
+                        % (first.capitalize(), "Llama decoder" if first == "kasuvik" else "Kasuvik and Llama decoders"), "dtype": key,
               "data": "synthetic", "layers": layers, "prefill_tokens": T, "prompt_len": args.prompt_len, "steps": steps, "sizes": {}}
     for width in [int(w) for w in args.design_sizes.split(",")]:
         if width not in DESIGN_SIZES:
             print("bench.py: unknown width %d for --design-sizes; known: %s" % (width, sorted(DESIGN_SIZES)))
             sys.exit(2)
         entry = {}
-        for name, cfg in zip(("kasuvik", "llama"), kasuvik_pair(width, layers)):
-            arch = "Kasuvik" if name == "kasuvik" else "LlamaForCausalLM"
+        designs = dict(zip(("kasuvik", "llama"), kasuvik_pair(width, layers)))
+        if first == "furapel":
+            designs = {"furapel": furapel_config(width, layers), **designs}
+        for name, cfg in designs.items():
+            arch = {"kasuvik": "Kasuvik", "furapel": "Furapel", "llama": "LlamaForCausalLM"}[name]
             tensors = random_tensors(arch, cfg, seed=0, dtype=dt, device="cuda:0")
             ec = EngineConfig(block_size=16, max_seq_len=limit, num_blocks=8 * limit // 16, max_num_seqs=8,
                               max_batched_tokens=max(4096, T + 64), dtype=args.dtype, max_logit_rows=64, beyond_max_position=True)
@@ -189,7 +221,9 @@ def design_main(args):
             del tensors
             V = eng.model.spec.vocab_size
             sec = prefill_run(eng, T, V)
-            flops = eng.model.step_flops(T, 1, T * (T + 1) // 2 if name == "llama" else T * min(T, DESIGN_SIZES[width][4]))
+            # (row, key) pairs a prompt's rows see: all earlier tokens, or a window's; Furapel's layers differ (its parts are
+            # asked with the full count: its attention layers weigh most)
+            flops = eng.model.step_flops(T, 1, T * min(T, DESIGN_SIZES[width][4]) if name == "kasuvik" else T * (T + 1) // 2)
             one = {"prefill_tok_s": round(T / sec, 1), "prefill_ms": round(sec * 1e3, 3),
                    "prefill_flops_frac": round(flops / sec / PEAK_FLOPS[key], 4)}
             for b in (1, 8):
@@ -200,8 +234,8 @@ def design_main(args):
             entry[name] = one
             del eng
             torch.cuda.empty_cache()
-        entry["prefill_ratio"] = round(entry["kasuvik"]["prefill_tok_s"] / entry["llama"]["prefill_tok_s"], 3)
-        entry["decode_b8_ratio"] = round(entry["kasuvik"]["decode_b8_tok_s"] / entry["llama"]["decode_b8_tok_s"], 3)
+        entry["prefill_ratio"] = round(entry[first]["prefill_tok_s"] / entry["llama"]["prefill_tok_s"], 3)
+        entry["decode_b8_ratio"] = round(entry[first]["decode_b8_tok_s"] / entry["llama"]["decode_b8_tok_s"], 3)
         record["sizes"][str(width)] = entry
     print(json.dumps(record), flush=True)
 
@@ -229,9 +263,10 @@ def main():
                     help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="tokens of the prefill measurement (2,048 in the record; other lengths for sweeps)")
-    ap.add_argument("--design", default="llama", choices=["llama", "kasuvik"],
+    ap.add_argument("--design", default="llama", choices=["llama", "kasuvik", "furapel"],
                     help="llama: the workload above (the default); kasuvik: prefill and decode of the Kasuvik decoder beside the "
-                         "Llama decoder at equal sizes (--design-sizes, --layers, --prefill-tokens, --prompt-len, --steps)")
+                         "Llama decoder at equal sizes; furapel: the same for the Furapel decoder beside both "
+                         "(--design-sizes, --layers, --prefill-tokens, --prompt-len, --steps)")
     ap.add_argument("--design-sizes", default="2048,4096", help="widths of the --design comparison (2048, 4096)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:

@@ -213,13 +213,21 @@ int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const floa
 int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* ig, int ldi,
                     const float* fg, int ldf, const float* i_bias, const float* f_bias, float cap, float q_scale, float* coef,
                     float* o, int ldo, float* s_state, float* n_state, float* m_state, const int* run_start,
-                    const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s);
+                    const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, int T, int max_run,
+                    hipStream_t s);
 // (moe.hip) a routed feed-forward: the choice of experts, and the experts' two products a row at a time
 int kvcm_moe_route(const float* logits, int ld, int E, int top, int* chosen, float* weight, int T, hipStream_t s);
 int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* chosen, void* act, int T, int K, int F, int top,
                 int E, hipStream_t s);
 int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* chosen, const float* weight, float* out, int T,
                   int F, int H, int top, int E, hipStream_t s);
+
+// (moe_grouped.hip) the routed feed-forward for many rows: pairs grouped by expert, tiles on the matrix cores
+int kvcm_moe_grouped_supported(int K, int F, int E);
+int kvcm_moe_grouped_max_tiles(int n, int E);
+int kvcm_moe_grouped(const void* h, int ldh, const void* w_up, const void* w_down, const int* chosen, const float* weight,
+                     int* order, int* tiles, void* act, float* y, float* out, int T, int K, int F, int H, int top, int E,
+                     hipStream_t s);
 
 // ---- recorded steps ---------------------------------------------------------------------------
 // A step program is the list of launches of one step, recorded once for a step shape and replayed

@@ -26,6 +26,20 @@ __device__ __forceinline__ float log_sigmoid(float z) { return z >= 0.f ? -log1p
 constexpr int kGateTile = 8;
 constexpr int kGateMaxPerLane = 4;      // dk up to 256 over 64 lanes
 
+// For steps with long runs the gates' logarithms of all rows are made first, in parallel: coef[row, head] = (li, lf, ., .);
+// the walk below then has no transcendental function but its three exponentials a token.
+__global__ void __launch_bounds__(256)
+    mlstm_gate_logs_kernel(const float* __restrict__ ig, int ldi, const float* __restrict__ fg, int ldf,
+                           const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
+                           float4* __restrict__ coef, long long n, int heads) {
+  const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const long long row = idx / heads;
+  const int head = static_cast<int>(idx % heads);
+  coef[idx] = float4{soft_cap(ig[row * ldi + head] + i_bias[head], cap), log_sigmoid(soft_cap(fg[row * ldf + head] + f_bias[head], cap)),
+                     0.f, 0.f};
+}
+
 // one wave per (sequence, head): coef[row, head] = (keep, take, 1 / den, m) for every row of the run
 __global__ void __launch_bounds__(kWave)
     mlstm_gates_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk,
@@ -33,7 +47,7 @@ __global__ void __launch_bounds__(kWave)
                        const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale,
                        float4* __restrict__ coef, float* __restrict__ n_state, float* __restrict__ m_state,
                        const int* __restrict__ run_start, const int* __restrict__ seq_start,
-                       const int* __restrict__ state_slots, int heads, int dk) {
+                       const int* __restrict__ state_slots, int heads, int dk, int logs_ready) {
   const int head = blockIdx.x, s = blockIdx.y, lane = threadIdx.x;
   const int r0 = run_start[s], r1 = run_start[s + 1];
   const int slot = state_slots[s];
@@ -58,8 +72,14 @@ __global__ void __launch_bounds__(kWave)
 #pragma unroll
     for (int t = 0; t < kGateTile; ++t) {
       const int row = t0 + t < r1 ? t0 + t : r1 - 1;
-      gi[t] = ig[size_t(row) * ldi + head];
-      gf[t] = fg[size_t(row) * ldf + head];
+      if (logs_ready) {
+        const float4 c = coef[size_t(row) * heads + head];
+        gi[t] = c.x;
+        gf[t] = c.y;
+      } else {
+        gi[t] = ig[size_t(row) * ldi + head];
+        gf[t] = fg[size_t(row) * ldf + head];
+      }
 #pragma unroll
       for (int e = 0; e < kGateMaxPerLane; ++e) {
         const int i = lane + e * kWave;
@@ -72,7 +92,8 @@ __global__ void __launch_bounds__(kWave)
 #pragma unroll
     for (int t = 0; t < kGateTile; ++t) {
       if (t0 + t >= r1) break;
-      const float li = soft_cap(gi[t] + ib, cap), lf = log_sigmoid(soft_cap(gf[t] + fb, cap));
+      const float li = logs_ready ? gi[t] : soft_cap(gi[t] + ib, cap);
+      const float lf = logs_ready ? gf[t] : log_sigmoid(soft_cap(gf[t] + fb, cap));
       const float m_new = fmaxf(lf + m, li);
       const float keep = expf(lf + m - m_new), take = expf(li - m_new);
       m = m_new;
@@ -193,12 +214,13 @@ using namespace kvcm;
 extern "C" {
 
 // q, k [T, heads*dk], v [T, heads*dv], ig, fg [T, heads] (the gates' projections without their biases), at their own
-// strides; i_bias, f_bias [heads]; coef: scratch of 4 T heads floats; o [T, >= heads*dv]; s_state [slots, heads, dk, dv],
+// strides; i_bias, f_bias [heads]; coef: scratch of 4 T heads floats (T: the step's rows, max_run: its longest run); o [T, >= heads*dv]; s_state [slots, heads, dk, dv],
 // n_state [slots, heads, dk], m_state [slots, heads]; all 32-bit.
 int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* ig, int ldi,
                     const float* fg, int ldf, const float* i_bias, const float* f_bias, float cap, float q_scale, float* coef,
                     float* o, int ldo, float* s_state, float* n_state, float* m_state, const int* run_start,
-                    const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, hipStream_t s) {
+                    const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, int T, int max_run,
+                    hipStream_t s) {
   if (S == 0) return 0;
   KVCM_REQUIRE(S > 0 && heads > 0 && dk > 0 && dv > 0, "mlstm_scan: bad sizes S=%d heads=%d dk=%d dv=%d", S, heads, dk, dv);
   KVCM_REQUIRE(dk <= kGateMaxPerLane * kWave, "mlstm_scan: a key size of %d is not supported (up to %d)", dk, kGateMaxPerLane * kWave);
@@ -209,8 +231,14 @@ int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const floa
                "mlstm_scan: row strides too small");
   KVCM_REQUIRE(coef && reinterpret_cast<uintptr_t>(coef) % 16 == 0, "mlstm_scan: the factors' scratch must be 16-byte aligned");
   float4* cf = reinterpret_cast<float4*>(coef);
+  const int logs_first = max_run >= 16 ? 1 : 0;      // long runs: the gates' logarithms of all T rows first, in parallel
+  if (logs_first) {
+    KVCM_REQUIRE(T > 0, "mlstm_scan: the row count is needed for runs of %d", max_run);
+    const long long n = static_cast<long long>(T) * heads;
+    mlstm_gate_logs_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, s>>>(ig, ldi, fg, ldf, i_bias, f_bias, cap, cf, n, heads);
+  }
   mlstm_gates_kernel<<<dim3(heads, S), kWave, 0, s>>>(q, ldq, k, ldk, ig, ldi, fg, ldf, i_bias, f_bias, cap, q_scale, cf, n_state,
-                                                      m_state, run_start, seq_start, state_slots, heads, dk);
+                                                      m_state, run_start, seq_start, state_slots, heads, dk, logs_first);
 #define KVCM_MLSTM(DKP, G, TILE)                                                                                             \
   {                                                                                                                          \
     const int col_blocks = (dv + 256 / G - 1) / (256 / G);                                                                   \

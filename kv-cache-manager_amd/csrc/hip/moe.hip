@@ -74,32 +74,54 @@ __device__ __forceinline__ void unpack16(const bf16_t* p, float* f) {
   f[6] = bf16_bits_to_float(v.w & 0xffffu); f[7] = bf16_bits_to_float(v.w >> 16);
 }
 
-// sum over k of xs[k] * w[k], w a stored row of K values, xs the row in LDS; the wave's lanes take pieces in turn
-template <class T>
-__device__ __forceinline__ float wave_dot(const float* xs, const T* w, int K, int lane, bool vec) {
+// CW sums at once: out[c] = sum over k of xs[k] * w[c * stride + k], c < CW (columns beyond ``cols`` repeat the last
+// one and are dropped by the caller), xs the row in LDS; a lane takes 16-byte pieces of every column's stored row in
+// turn, so that CW loads are on their way per trip and the row's values are read from LDS once for all of them.
+template <class T, int CW>
+__device__ __forceinline__ void wave_dots(const float* xs, const T* w, size_t stride, int cols, int K, int lane, bool vec,
+                                          float* out) {
   constexpr int N = Piece<T>::N;
-  float acc = 0.f;
-  if (vec) {
-    for (int k = lane * N; k < K; k += kWave * N) {
-      float f[N];
-      unpack16(w + k, f);
+  float acc[CW];
+  const T* wc[CW];
 #pragma unroll
-      for (int e = 0; e < N; ++e) acc = fmaf(xs[k + e], f[e], acc);
+  for (int c = 0; c < CW; ++c) {
+    acc[c] = 0.f;
+    wc[c] = w + size_t(c < cols ? c : cols - 1) * stride;
+  }
+  if (vec) {
+#pragma unroll 2
+    for (int k = lane * N; k < K; k += kWave * N) {
+      float f[CW][N];
+#pragma unroll
+      for (int c = 0; c < CW; ++c) unpack16(wc[c] + k, f[c]);
+      float xv[N];
+#pragma unroll
+      for (int e = 0; e < N; e += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(xs + k + e);
+        xv[e] = v.x; xv[e + 1] = v.y; xv[e + 2] = v.z; xv[e + 3] = v.w;
+      }
+#pragma unroll
+      for (int c = 0; c < CW; ++c)
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[c] = fmaf(xv[e], f[c][e], acc[c]);
     }
   } else {
-    for (int k = lane; k < K; k += kWave) acc = fmaf(xs[k], load_f(w + k), acc);
+    for (int k = lane; k < K; k += kWave) {
+      const float x = xs[k];
+#pragma unroll
+      for (int c = 0; c < CW; ++c) acc[c] = fmaf(x, load_f(wc[c] + k), acc[c]);
+    }
   }
-  return wave_sum(acc);
+#pragma unroll
+  for (int c = 0; c < CW; ++c) out[c] = wave_sum(acc[c]);
 }
 
-constexpr int kMoeCols = 32;      // output columns of a workgroup (8 a wave)
-
-// grid (T * top, column blocks).  h [T, K] in T; w_up [E, F, K]; act [T * top, F].
-template <class T>
+// grid (T * top, column blocks of 4 CW).  h [T, K] in T; w_up [E, F, K]; act [T * top, F].
+template <class T, int CW>
 __global__ void __launch_bounds__(256)
     moe_up_kernel(const T* __restrict__ h, int ldh, const T* __restrict__ w_up, const int* __restrict__ chosen,
                   T* __restrict__ act, int K, int F, int top, int E) {
-  extern __shared__ float xs[];
+  extern __shared__ __attribute__((aligned(16))) float xs[];
   const int item = blockIdx.x, row = item / top;
   const int e = chosen[item];
   for (int k = threadIdx.x; k < K; k += 256) xs[k] = load_f(h + size_t(row) * ldh + k);
@@ -107,35 +129,54 @@ __global__ void __launch_bounds__(256)
   if (e < 0 || e >= E) return;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const bool vec = K % Piece<T>::N == 0;
-  const T* w = w_up + size_t(e) * F * K;
-  for (int c = blockIdx.y * kMoeCols + wave; c < min(F, (blockIdx.y + 1) * kMoeCols); c += 256 / kWave) {
-    const float z = wave_dot(xs, w + size_t(c) * K, K, lane, vec);
-    const float r = fmaxf(z, 0.f);
-    if (lane == 0) store_f(act + size_t(item) * F + c, r * r);
-  }
+  const int c0 = (blockIdx.y * 4 + wave) * CW;
+  if (c0 >= F) return;
+  const int cols = F - c0 < CW ? F - c0 : CW;
+  float z[CW];
+  wave_dots<T, CW>(xs, w_up + (size_t(e) * F + c0) * K, K, cols, K, lane, vec, z);
+  if (lane == 0)
+    for (int c = 0; c < cols; ++c) {
+      const float r = fmaxf(z[c], 0.f);
+      store_f(act + size_t(item) * F + c0 + c, r * r);
+    }
 }
 
-// grid (T, column blocks).  act [T * top, F] in T; w_down [E, H, F]; out [T, H] 32-bit.
-template <class T>
+// grid (T, column blocks of 4 CW).  act [T * top, F] in T; w_down [E, H, F]; out [T, H] 32-bit.
+template <class T, int CW>
 __global__ void __launch_bounds__(256)
     moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down, const int* __restrict__ chosen,
                     const float* __restrict__ weight, float* __restrict__ out, int F, int H, int top, int E) {
-  extern __shared__ float xs[];      // [top][F]
+  extern __shared__ __attribute__((aligned(16))) float xs[];      // [top][F4], F4: F rounded up to 4
   const int row = blockIdx.x;
-  for (int k = threadIdx.x; k < top * F; k += 256) xs[k] = load_f(act + size_t(row) * top * F + k);
+  const int F4 = (F + 3) & ~3;
+  for (int k = threadIdx.x; k < top * F; k += 256) xs[(k / F) * F4 + k % F] = load_f(act + size_t(row) * top * F + k);
   __syncthreads();
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const bool vec = F % Piece<T>::N == 0;
-  for (int c = blockIdx.y * kMoeCols + wave; c < min(H, (blockIdx.y + 1) * kMoeCols); c += 256 / kWave) {
-    float acc = 0.f;
-    for (int s = 0; s < top; ++s) {
-      const int e = chosen[size_t(row) * top + s];
-      if (e < 0 || e >= E) continue;
-      const float z = wave_dot(xs + s * F, w_down + (size_t(e) * H + c) * F, F, lane, vec);
-      acc = fmaf(weight[size_t(row) * top + s], z, acc);
-    }
-    if (lane == 0) out[size_t(row) * H + c] = acc;
+  const int c0 = (blockIdx.y * 4 + wave) * CW;
+  if (c0 >= H) return;
+  const int cols = H - c0 < CW ? H - c0 : CW;
+  float acc[CW];
+#pragma unroll
+  for (int c = 0; c < CW; ++c) acc[c] = 0.f;
+  for (int s = 0; s < top; ++s) {
+    const int e = chosen[size_t(row) * top + s];
+    if (e < 0 || e >= E) continue;
+    float z[CW];
+    wave_dots<T, CW>(xs + s * F4, w_down + (size_t(e) * H + c0) * F, F, cols, F, lane, vec, z);
+    const float g = weight[size_t(row) * top + s];
+#pragma unroll
+    for (int c = 0; c < CW; ++c) acc[c] = fmaf(g, z[c], acc[c]);
   }
+  if (lane == 0)
+    for (int c = 0; c < cols; ++c) out[size_t(row) * H + c0 + c] = acc[c];
+}
+
+// columns a wave takes at once: as many as still leave the chip a few workgroups per CU
+inline int moe_cols_per_wave(long long rows, int cols) {
+  for (int cw = 4; cw > 1; cw /= 2)
+    if (rows * ((cols + 4 * cw - 1) / (4 * cw)) >= 512) return cw;
+  return 1;
 }
 
 }  // namespace kvcm
@@ -157,17 +198,19 @@ int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* 
                 int E, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && K > 0 && F > 0 && top > 0 && E > 0 && ldh >= K, "moe_up: bad sizes");
-  KVCM_REQUIRE(static_cast<long long>(T) * top < (1ll << 31) && (F + kMoeCols - 1) / kMoeCols <= 65535, "moe_up: too many rows or columns");
+  KVCM_REQUIRE(static_cast<long long>(T) * top < (1ll << 31) && (F + 3) / 4 <= 65535, "moe_up: too many rows or columns");
   KVCM_REQUIRE(K * sizeof(float) <= 64 * 1024, "moe_up: rows of %d values do not fit the local memory", K);
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(w_up) % 16 == 0, "moe_up: weights must be 16-byte aligned");
-  const dim3 grid(T * top, (F + kMoeCols - 1) / kMoeCols);
-  if (dtype == kF32)
-    moe_up_kernel<float><<<grid, 256, K * sizeof(float), s>>>(static_cast<const float*>(h), ldh, static_cast<const float*>(w_up),
-                                                             chosen, static_cast<float*>(act), K, F, top, E);
-  else if (dtype == kBF16)
-    moe_up_kernel<bf16_t><<<grid, 256, K * sizeof(float), s>>>(static_cast<const bf16_t*>(h), ldh, static_cast<const bf16_t*>(w_up),
-                                                              chosen, static_cast<bf16_t*>(act), K, F, top, E);
-  else KVCM_REQUIRE(false, "moe_up: unknown dtype %d", dtype);
+  KVCM_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_up: unknown dtype %d", dtype);
+  const int cw = moe_cols_per_wave(static_cast<long long>(T) * top, F);
+  const dim3 grid(T * top, (F + 4 * cw - 1) / (4 * cw));
+  const size_t lds = K * sizeof(float);
+#define KVCM_MOE_UP(TT, CW)                                                                                              \
+  moe_up_kernel<TT, CW><<<grid, 256, lds, s>>>(static_cast<const TT*>(h), ldh, static_cast<const TT*>(w_up), chosen,     \
+                                               static_cast<TT*>(act), K, F, top, E)
+  if (dtype == kF32) { if (cw == 4) KVCM_MOE_UP(float, 4); else if (cw == 2) KVCM_MOE_UP(float, 2); else KVCM_MOE_UP(float, 1); }
+  else { if (cw == 4) KVCM_MOE_UP(bf16_t, 4); else if (cw == 2) KVCM_MOE_UP(bf16_t, 2); else KVCM_MOE_UP(bf16_t, 1); }
+#undef KVCM_MOE_UP
   return launch_status("moe_up");
 }
 
@@ -176,18 +219,19 @@ int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* cho
                   int F, int H, int top, int E, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && H > 0 && F > 0 && top > 0 && E > 0, "moe_down: bad sizes");
-  KVCM_REQUIRE(static_cast<size_t>(top) * F * sizeof(float) <= 64 * 1024, "moe_down: %d activations of %d values do not fit the local memory", top, F);
+  const size_t lds = static_cast<size_t>(top) * ((F + 3) & ~3) * sizeof(float);
+  KVCM_REQUIRE(lds <= 64 * 1024, "moe_down: %d activations of %d values do not fit the local memory", top, F);
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(w_down) % 16 == 0, "moe_down: weights must be 16-byte aligned");
-  KVCM_REQUIRE((H + kMoeCols - 1) / kMoeCols <= 65535, "moe_down: too many columns");
-  const dim3 grid(T, (H + kMoeCols - 1) / kMoeCols);
-  const size_t lds = static_cast<size_t>(top) * F * sizeof(float);
-  if (dtype == kF32)
-    moe_down_kernel<float><<<grid, 256, lds, s>>>(static_cast<const float*>(act), static_cast<const float*>(w_down), chosen, weight,
-                                                 out, F, H, top, E);
-  else if (dtype == kBF16)
-    moe_down_kernel<bf16_t><<<grid, 256, lds, s>>>(static_cast<const bf16_t*>(act), static_cast<const bf16_t*>(w_down), chosen,
-                                                  weight, out, F, H, top, E);
-  else KVCM_REQUIRE(false, "moe_down: unknown dtype %d", dtype);
+  KVCM_REQUIRE((H + 3) / 4 <= 65535, "moe_down: too many columns");
+  KVCM_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_down: unknown dtype %d", dtype);
+  const int cw = moe_cols_per_wave(T, H);
+  const dim3 grid(T, (H + 4 * cw - 1) / (4 * cw));
+#define KVCM_MOE_DOWN(TT, CW)                                                                                                \
+  moe_down_kernel<TT, CW><<<grid, 256, lds, s>>>(static_cast<const TT*>(act), static_cast<const TT*>(w_down), chosen, weight, \
+                                                 out, F, H, top, E)
+  if (dtype == kF32) { if (cw == 4) KVCM_MOE_DOWN(float, 4); else if (cw == 2) KVCM_MOE_DOWN(float, 2); else KVCM_MOE_DOWN(float, 1); }
+  else { if (cw == 4) KVCM_MOE_DOWN(bf16_t, 4); else if (cw == 2) KVCM_MOE_DOWN(bf16_t, 2); else KVCM_MOE_DOWN(bf16_t, 1); }
+#undef KVCM_MOE_DOWN
   return launch_status("moe_down");
 }
 

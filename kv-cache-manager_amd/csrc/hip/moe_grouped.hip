@@ -1,0 +1,203 @@
+// The routed feed-forward for steps with many rows (bfloat16): the (row, slot) pairs are grouped by their expert and
+// every expert's group is multiplied with that expert's matrices in tiles on the matrix cores, so that an expert's
+// weights are read once per tile of 128 pairs and not once per pair.
+//
+//   moe_group      pairs p = row * top + slot, grouped by chosen[p]: order[] lists the pairs expert by expert, tiles[]
+//                  lists (expert, first place in order, pairs) for every stretch of up to 128 pairs of one expert, with
+//                  the number of tiles in front.  One workgroup; places inside a group are handed out by an atomic
+//                  counter in LDS, so the order inside a group may differ from run to run, which changes no result: a
+//                  pair's row of a tile is computed from that row alone.
+//   moe_grouped    UP:   act[place, :] = square(relu(W_up[e] h[row of the pair]))           (bfloat16, in grouped order)
+//                  DOWN: y[pair, :]   = weight[pair] * W_down[e] act[place, :]               (32-bit, by pair)
+//                  Tile 128 pairs x 128 columns per workgroup of four waves (64 x 64 each: 4 x 4 matrix instructions of
+//                  16 x 16 x 32), K advanced 64 at a time through LDS, the next 64 on their way in registers meanwhile.
+//   moe_combine    out[row, :] = sum over the row's slots, in slot order, of y[row * top + slot, :]
+#include "common.h"
+#include "kvcm_hip.h"
+
+namespace kvcm {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int kGM = 128, kGN = 128, kGK = 64, kGPitch = kGK + 8;      // a row pitch of 144 bytes: 16 rows meet no bank twice
+
+__global__ void __launch_bounds__(1024)
+    moe_group_kernel(const int* __restrict__ chosen, int n, int E, int* __restrict__ order, int* __restrict__ tiles, int max_tiles) {
+  extern __shared__ int sh[];      // count / cursor [E], base [E]
+  int* cnt = sh;
+  int* base = sh + E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < n; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      base[e] = at;
+      for (int r = 0; r < cnt[e] && nt < max_tiles; r += kGM) {
+        tiles[1 + 3 * nt] = e;
+        tiles[2 + 3 * nt] = at + r;
+        tiles[3 + 3 * nt] = cnt[e] - r < kGM ? cnt[e] - r : kGM;
+        ++nt;
+      }
+      at += cnt[e];
+      cnt[e] = 0;
+    }
+    tiles[0] = nt;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < n; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e >= 0 && e < E) order[base[e] + atomicAdd(&cnt[e], 1)] = p;
+  }
+}
+
+template <bool UP>
+__global__ void __launch_bounds__(256)
+    moe_grouped_kernel(const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, const int* __restrict__ order,
+                       const int* __restrict__ tiles, int top, void* __restrict__ out, const float* __restrict__ weight, int N,
+                       int K) {
+  __shared__ __attribute__((aligned(16))) uint16_t As[kGM][kGPitch];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[kGN][kGPitch];
+  __shared__ int pair_of[kGM];
+  const int tile = blockIdx.x;
+  if (tile >= tiles[0]) return;
+  const int e = tiles[1 + 3 * tile], p0 = tiles[2 + 3 * tile], rows = tiles[3 + 3 * tile];
+  const int n0 = blockIdx.y * kGN;
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  if (tid < kGM) pair_of[tid] = order[p0 + (tid < rows ? tid : 0)];
+  __syncthreads();
+  // the four 16-byte pieces a thread stages of each operand: rows tid / 8 + 32 q, k offset (tid % 8) * 8
+  const int kk = (tid % 8) * 8;
+  const uint16_t* arow[4];
+  const uint16_t* brow[4];
+  bool aok[4], bok[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = tid / 8 + 32 * q;
+    aok[q] = r < rows;
+    const long long src = UP ? pair_of[r] / top : p0 + (aok[q] ? r : 0);
+    arow[q] = A + src * lda + kk;
+    const int c = n0 + r;
+    bok[q] = c < N;
+    brow[q] = W + (static_cast<long long>(e) * N + (bok[q] ? c : N - 1)) * K + kk;
+  }
+  uint4 areg[4], breg[4];
+  auto request = [&](int k0) {      // unconditional loads from clamped places, masked afterwards
+    const bool kin = k0 + kk < K;      // K is a multiple of 8: a piece lies inside or outside
+    const int off = kin ? k0 : 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint4 a = *reinterpret_cast<const uint4*>(arow[q] + off);
+      const uint4 b = *reinterpret_cast<const uint4*>(brow[q] + off);
+      areg[q] = (kin && aok[q]) ? a : uint4{0u, 0u, 0u, 0u};
+      breg[q] = (kin && bok[q]) ? b : uint4{0u, 0u, 0u, 0u};
+    }
+  };
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int wm = wave / 2, wn = wave % 2;
+  const int frow = lane % 16, fk = (lane / 16) * 8;
+  request(0);
+  for (int k0 = 0; k0 < K; k0 += kGK) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      *reinterpret_cast<uint4*>(&As[tid / 8 + 32 * q][kk]) = areg[q];
+      *reinterpret_cast<uint4*>(&Bs[tid / 8 + 32 * q][kk]) = breg[q];
+    }
+    __syncthreads();
+    if (k0 + kGK < K) request(k0 + kGK);
+#pragma unroll
+    for (int ks = 0; ks < kGK / 32; ++ks) {
+      bf16x8 a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const bf16x8*>(&As[wm * 64 + i * 16 + frow][ks * 32 + fk]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const bf16x8*>(&Bs[wn * 64 + j * 16 + frow][ks * 32 + fk]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  // accumulator layout: a lane holds column lane % 16 and rows 4 * (lane / 16) + r of each 16 x 16 tile
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = wm * 64 + i * 16 + (lane / 16) * 4 + r;
+      if (m >= rows) continue;
+      const int pair = pair_of[m];
+      const float g = UP ? 1.f : weight[pair];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int c = n0 + wn * 64 + j * 16 + lane % 16;
+        if (c >= N) continue;
+        const float v = acc[i][j][r];
+        if (UP) {
+          const float z = fmaxf(v, 0.f);
+          static_cast<uint16_t*>(out)[static_cast<long long>(p0 + m) * N + c] = float_to_bf16_bits(z * z);
+        } else {
+          static_cast<float*>(out)[static_cast<long long>(pair) * N + c] = g * v;
+        }
+      }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+    moe_combine_kernel(const float* __restrict__ y, float* __restrict__ out, long long n, int H, int top) {
+  for (long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x; idx < n; idx += static_cast<long long>(gridDim.x) * 256) {
+    const long long row = idx / H;
+    const int c = static_cast<int>(idx % H);
+    float acc = 0.f;
+    for (int s = 0; s < top; ++s) acc += y[(row * top + s) * H + c];
+    out[idx] = acc;
+  }
+}
+
+}  // namespace kvcm
+
+using namespace kvcm;
+
+extern "C" {
+
+// Does the grouped form take these sizes?  (bfloat16; rows of 16-byte pieces)
+int kvcm_moe_grouped_supported(int K, int F, int E) { return K > 0 && F > 0 && K % 8 == 0 && F % 8 == 0 && E > 0 && E <= 4096; }
+
+// Tiles a step of n pairs over E experts can have at most.
+int kvcm_moe_grouped_max_tiles(int n, int E) { return (n + kGM - 1) / kGM + E; }
+
+// h [T, K] bfloat16; w_up [E, F, K], w_down [E, H, F] bfloat16; chosen [T * top], weight [T * top]; work memory:
+// order [T * top] and tiles [3 * max_tiles + 1] (int32), act [T * top, F] (bfloat16), y [T * top, H] (32-bit); out [T, H] 32-bit.
+int kvcm_moe_grouped(const void* h, int ldh, const void* w_up, const void* w_down, const int* chosen, const float* weight,
+                     int* order, int* tiles, void* act, float* y, float* out, int T, int K, int F, int H, int top, int E,
+                     hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && top > 0 && H > 0 && ldh >= K, "moe_grouped: bad sizes");
+  KVCM_REQUIRE(kvcm_moe_grouped_supported(K, F, E), "moe_grouped: sizes K=%d F=%d experts=%d are not supported", K, F, E);
+  KVCM_REQUIRE(static_cast<long long>(T) * top < (1ll << 30), "moe_grouped: too many rows");
+  KVCM_REQUIRE(ldh % 8 == 0 && reinterpret_cast<uintptr_t>(h) % 16 == 0 && reinterpret_cast<uintptr_t>(w_up) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(w_down) % 16 == 0 && reinterpret_cast<uintptr_t>(act) % 16 == 0,
+               "moe_grouped: operands must be 16-byte aligned");
+  const int n = T * top, max_tiles = kvcm_moe_grouped_max_tiles(n, E);
+  KVCM_REQUIRE((F + kGN - 1) / kGN <= 65535 && (H + kGN - 1) / kGN <= 65535, "moe_grouped: too many columns");
+  moe_group_kernel<<<1, 1024, 2 * E * sizeof(int), s>>>(chosen, n, E, order, tiles, max_tiles);
+  moe_grouped_kernel<true><<<dim3(max_tiles, (F + kGN - 1) / kGN), 256, 0, s>>>(
+      static_cast<const uint16_t*>(h), ldh, static_cast<const uint16_t*>(w_up), order, tiles, top, act, nullptr, F, K);
+  moe_grouped_kernel<false><<<dim3(max_tiles, (H + kGN - 1) / kGN), 256, 0, s>>>(
+      static_cast<const uint16_t*>(act), F, static_cast<const uint16_t*>(w_down), order, tiles, top, y, weight, H, F);
+  const long long total = static_cast<long long>(T) * H;
+  const long long blocks = (total + 255) / 256;
+  moe_combine_kernel<<<static_cast<unsigned>(blocks > 16384 ? 16384 : blocks), 256, 0, s>>>(y, out, total, H, top);
+  return launch_status("moe_grouped");
+}
+
+}  // extern "C"

@@ -109,6 +109,7 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_moe_route),
     KVCM_ENTRY(kvcm_moe_up),
     KVCM_ENTRY(kvcm_moe_down),
+    KVCM_ENTRY(kvcm_moe_grouped),
     KVCM_ENTRY(kvcm_pool_update),
     KVCM_ENTRY(kvcm_attention_window_pool),
     KVCM_ENTRY(kvcm_attention_window_pool_tiles),

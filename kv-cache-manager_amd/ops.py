@@ -101,10 +101,13 @@ def _declare(lib):
     fn("kvcm_scale_rows", vp, C.c_longlong, f, vp)
     fn("kvcm_head_gate", vp, i, i, vp, i, i, i, i, vp)
     fn("kvcm_rms_groups", vp, i, i, i, i, vp, f, i, vp)
-    fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, vp)
+    fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_moe_route", vp, i, i, i, vp, vp, i, vp)
     fn("kvcm_moe_up", vp, i, i, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_moe_down", vp, i, vp, vp, vp, vp, i, i, i, i, i, vp)
+    fn("kvcm_moe_grouped_supported", i, i, i)
+    fn("kvcm_moe_grouped_max_tiles", i, i)
+    fn("kvcm_moe_grouped", vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_pool_update", vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp)
     fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
@@ -1363,7 +1366,7 @@ def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, co
     _call("kvcm_mlstm_scan", _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(gate_in), gate_in.stride(0),
           _ptr(gate_keep), gate_keep.stride(0), _ptr(in_bias), _ptr(keep_bias), float(cap), float(q_scale), _ptr(coef), _ptr(o),
           o.stride(0), _ptr(s_state), _ptr(n_state), _ptr(m_state), _ptr(step.run_start), _ptr(step.seq_start),
-          _ptr(step.state_slots), step.seqs, heads, dk, dv, _stream())
+          _ptr(step.state_slots), step.seqs, heads, dk, dv, T, int(step.max_run), _stream())
     return o
 
 
@@ -1395,4 +1398,37 @@ def moe_rows(h, w_up, w_down, chosen, weight, act, out):
     _need(weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == tuple(chosen.shape), "weight must match chosen")
     _call("kvcm_moe_up", _ptr(h), _DT[h.dtype], h.stride(0), _ptr(w_up), _ptr(chosen), _ptr(act), T, K, F, top, E, _stream())
     _call("kvcm_moe_down", _ptr(act), _DT[act.dtype], _ptr(w_down), _ptr(chosen), _ptr(weight), _ptr(out), T, F, H, top, E, _stream())
+    return out
+
+
+def moe_grouped_supported(K, F, E, dtype):
+    """Does the grouped form of the routed feed-forward (tiles on the matrix cores) take these sizes?"""
+    return dtype == torch.bfloat16 and bool(lib().kvcm_moe_grouped_supported(int(K), int(F), int(E)))
+
+
+def moe_grouped_tiles(pairs, E):
+    """int32 values of work memory that ``moe_grouped`` needs for its list of tiles."""
+    return 3 * lib().kvcm_moe_grouped_max_tiles(int(pairs), int(E)) + 1
+
+
+def moe_grouped(h, w_up, w_down, chosen, weight, order, tiles, act, y, out):
+    """As ``moe_rows``, for steps with many rows (bfloat16): the (row, slot) pairs grouped by expert and multiplied in tiles
+    on the matrix cores.  Work memory: order int32 [T * top], tiles int32 [moe_grouped_tiles], act [T * top, F],
+    y float32 [T * top, H]."""
+    T, K = h.shape
+    E, F, _ = w_up.shape
+    H, top = w_down.shape[1], chosen.shape[1]
+    _rows2d(h, "h")
+    _need(h.is_cuda and h.dtype == w_up.dtype == w_down.dtype == act.dtype == torch.bfloat16, "moe_grouped takes bfloat16 operands")
+    _need(w_up.is_contiguous() and w_down.is_contiguous() and tuple(w_up.shape) == (E, F, K) and tuple(w_down.shape) == (E, H, F),
+          "moe_grouped: expert weights must be [E, F, K] and [E, H, F]")
+    _need(act.is_contiguous() and act.shape[0] >= T * top and act.shape[1] == F, "act must be [T * top, F]")
+    _need(y.dtype == torch.float32 and y.is_contiguous() and y.shape[0] >= T * top and y.shape[1] == H, "y must be float32 [T * top, H]")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H), "out must be float32 [T, H]")
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.shape[0] >= T, "chosen must be int32 [T, top]")
+    _need(weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == tuple(chosen.shape), "weight must match chosen")
+    _i32(order, "order", T * top)
+    _i32(tiles, "tiles", moe_grouped_tiles(T * top, E))
+    _call("kvcm_moe_grouped", _ptr(h), h.stride(0), _ptr(w_up), _ptr(w_down), _ptr(chosen), _ptr(weight), _ptr(order), _ptr(tiles),
+          _ptr(act), _ptr(y), _ptr(out), T, K, F, H, top, E, _stream())
     return out

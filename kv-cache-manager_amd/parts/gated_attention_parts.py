@@ -9,6 +9,7 @@ import math
 import torch
 
 from ..registry import MIXERS, POSITIONS
+from . import paged_attention
 from .base import KVCacheNeed, Mixer, ParamSpec, PartSpec, PositionEncoding
 from .chain_norm_parts import f32_params, linear32
 
@@ -49,6 +50,11 @@ class HalfSplitRotary(PositionEncoding):
         self.freqs, self.factor = rescaled_frequencies(self.dims, params["base"], params.get("scaling")) if self.dims else ([], 1.0)
         self._device_freqs = None
 
+    def bind(self, tensors):
+        super().bind(tensors)
+        if self.dims and self.ctx.device.type == "cuda":      # made once, here: a step allocates nothing
+            self._device_freqs = torch.tensor(self.freqs, dtype=torch.float64, device=self.ctx.device)
+
     def pairs_table(self, step):
         """factor * (cos, sin) of every row's angles, float32 [rows, dims/2, 2]; made by the step's first layer that asks,
         read by the others with the same frequencies."""
@@ -78,9 +84,13 @@ def _pad_rows(t, multiple=16):
 
 
 def _attend(mixer, step, q, attn, kc, vc, g, nh, nkv, d, dv, scale, window):
-    """Steps with runs of positions take the matrix-core kernel where it has the head shape, others one (row, head) per
-    workgroup."""
+    """Keys and values of one size, no window, bfloat16: the kernels every attention over paged keys and values takes
+    (parts/paged_attention.py: partitioned for single rows, tiled for runs of positions).  Otherwise the window
+    attention's: steps with runs of positions take its matrix-core kernel where it has the head shape, others one
+    (row, head) per workgroup."""
     ops = mixer.ctx.ops
+    if d == dv and window == 0 and attn.dtype == torch.bfloat16 and d % 8 == 0 and d <= 256:
+        return paged_attention.attend(step, ops, q, attn, kc, vc, g, nh, nkv, d, scale, 0)
     if step.max_run > 1 and ops.attention_window_pool_tiles_supported(d, dv, attn.dtype, kc.shape[2]):
         ops.attention_window_pool_tiles(q, attn, kc, vc, None, None, step.tables(g), step.table_stride(g), step.run_start,
                                         step.seq_start, step.seqs, step.max_run, nh, nkv, d, dv, scale, window, 0)
@@ -185,7 +195,9 @@ class LatentAttention(Mixer):
         return KVCacheNeed(1, self.r, self.params.get("window", 0), value_dim=self.r)
 
     def flops(self, rows, attended=0):
-        return super().flops(rows) + 4.0 * attended * self.r * self.nh
+        window = self.params.get("window", 0)
+        seen = min(attended, rows * window) if window else attended      # a row sees at most its window
+        return super().flops(rows) + 4.0 * seen * self.r * self.nh
 
     def forward(self, step, h):
         ops, p, w = self.ctx.ops, self.params, self.w

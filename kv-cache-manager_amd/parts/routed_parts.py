@@ -18,6 +18,8 @@ class RoutedExperts(FeedForward):
     (a pattern for an expert's prefix, default "e{}."), up, down (names after it).  The result is 32-bit."""
 
     capturable = True
+    # rows from which a bfloat16 step groups its (row, slot) pairs by expert; below, every pair streams its expert's rows itself
+    GROUPED_MIN_ROWS = 16
 
     def param_specs(self):
         H, p, pre = self.ctx.hidden_size, self.params, self.prefix
@@ -53,6 +55,13 @@ class RoutedExperts(FeedForward):
         chosen = step.ws("routed_chosen", (T, top), torch.int32)
         weight = step.ws("routed_weight", (T, top), torch.float32)
         ops.moe_route(logits, E, top, chosen, weight, rows=T)
+        H = self.ctx.hidden_size
         act = step.ws("routed_act", (T, top * F)).view(T * top, F)
-        out = step.ws("routed_out", (T, self.ctx.hidden_size), torch.float32)
+        out = step.ws("routed_out", (T, H), torch.float32)
+        if T >= self.GROUPED_MIN_ROWS and ops.moe_grouped_supported(H, F, E, act.dtype) and h.stride(0) % 8 == 0:
+            # many rows: the pairs grouped by expert, tiles on the matrix cores, every expert's weights read once per tile
+            order = step.ws("routed_order", (T, top), torch.int32)
+            tiles = step.flat("routed_tiles", ops.moe_grouped_tiles(max(T, step.limits.max_tokens if step.limits else T) * top, E), torch.int32)
+            y = step.ws("routed_y", (T, top * H), torch.float32).view(T * top, H)
+            return ops.moe_grouped(h, w["w_up"], w["w_down"], chosen, weight, order, tiles, act, y, out)
         return ops.moe_rows(h, w["w_up"], w["w_down"], chosen, weight, act, out)
