@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(256)
       const int tl = t < (t_lo / 8) * 8 ? (t_lo / 8) * 8 : t;
       const int tc = tl <= p_last ? tl : (p_last / 8) * 8, ccl = cc < dv ? cc : dv - 1;
       uint4 v = *reinterpret_cast<const uint4*>(vcache + ((size_t(table[tc / B]) * nkv + kvh) * dv + ccl) * B + tc % B);
-      v = keep_first_bf16(v, p_last + 1 - t < 8 ? p_last + 1 - t : 8);      // beyond the newest token: whatever was there
+      v = keep_first_bf16(v, p_last + 1 - tc < 8 ? p_last + 1 - tc : 8);      // beyond the newest token: whatever was there (counted from the piece that was read)
       vreg[qq] = cc < dv ? v : uint4{0u, 0u, 0u, 0u};
     }
   };

@@ -40,7 +40,9 @@ __global__ void __launch_bounds__(256)
                      0.f, 0.f};
 }
 
-// one wave per (sequence, head): coef[row, head] = (keep, take, 1 / den, m) for every row of the run
+// one wave per (sequence, head): coef[row, head] = (keep, take, 1 / den, m) for every row of the run.  PER: key entries
+// a lane carries (dk <= 64 PER).  The values of the next eight tokens are on their way while the current eight are walked.
+template <int PER>
 __global__ void __launch_bounds__(kWave)
     mlstm_gates_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk,
                        const float* __restrict__ ig, int ldi, const float* __restrict__ fg, int ldf,
@@ -59,57 +61,69 @@ __global__ void __launch_bounds__(kWave)
   float* nst = n_state + (size_t(slot) * heads + head) * dk;
   float* mst = m_state + size_t(slot) * heads + head;
   const bool fresh = seq_start[s] == 0;
-  float N[kGateMaxPerLane];
+  float N[PER];
 #pragma unroll
-  for (int e = 0; e < kGateMaxPerLane; ++e) {
+  for (int e = 0; e < PER; ++e) {
     const int i = lane + e * kWave;
     N[e] = (i < dk && !fresh) ? nst[i] : 0.f;
   }
   float m = fresh ? 0.f : *mst;
   const float ib = i_bias[head], fb = f_bias[head];
-  for (int t0 = r0; t0 < r1; t0 += kGateTile) {
-    float qv[kGateTile][kGateMaxPerLane], kv[kGateTile][kGateMaxPerLane], gi[kGateTile], gf[kGateTile];
+  float qv[2][kGateTile][PER], kv[2][kGateTile][PER], gi[2][kGateTile], gf[2][kGateTile];
+  auto request = [&](int t0, int buf) {      // unconditional loads from clamped places, masked afterwards
 #pragma unroll
     for (int t = 0; t < kGateTile; ++t) {
       const int row = t0 + t < r1 ? t0 + t : r1 - 1;
       if (logs_ready) {
         const float4 c = coef[size_t(row) * heads + head];
-        gi[t] = c.x;
-        gf[t] = c.y;
+        gi[buf][t] = c.x;
+        gf[buf][t] = c.y;
       } else {
-        gi[t] = ig[size_t(row) * ldi + head];
-        gf[t] = fg[size_t(row) * ldf + head];
+        gi[buf][t] = ig[size_t(row) * ldi + head];
+        gf[buf][t] = fg[size_t(row) * ldf + head];
       }
 #pragma unroll
-      for (int e = 0; e < kGateMaxPerLane; ++e) {
+      for (int e = 0; e < PER; ++e) {
         const int i = lane + e * kWave;
         const size_t col = size_t(head) * dk + (i < dk ? i : dk - 1);
         const float a = q[size_t(row) * ldq + col], b = k[size_t(row) * ldk + col];
-        qv[t][e] = i < dk ? a * q_scale : 0.f;
-        kv[t][e] = i < dk ? b : 0.f;
+        qv[buf][t][e] = i < dk ? a * q_scale : 0.f;
+        kv[buf][t][e] = i < dk ? b : 0.f;
       }
     }
+  };
+  auto walk = [&](int t0, int buf) {
 #pragma unroll
     for (int t = 0; t < kGateTile; ++t) {
       if (t0 + t >= r1) break;
-      const float li = logs_ready ? gi[t] : soft_cap(gi[t] + ib, cap);
-      const float lf = logs_ready ? gf[t] : log_sigmoid(soft_cap(gf[t] + fb, cap));
+      const float li = logs_ready ? gi[buf][t] : soft_cap(gi[buf][t] + ib, cap);
+      const float lf = logs_ready ? gf[buf][t] : log_sigmoid(soft_cap(gf[buf][t] + fb, cap));
       const float m_new = fmaxf(lf + m, li);
       const float keep = expf(lf + m - m_new), take = expf(li - m_new);
       m = m_new;
       float nq = 0.f;
 #pragma unroll
-      for (int e = 0; e < kGateMaxPerLane; ++e) {
-        N[e] = fmaf(keep, N[e], take * kv[t][e]);
-        nq = fmaf(N[e], qv[t][e], nq);
+      for (int e = 0; e < PER; ++e) {
+        N[e] = fmaf(keep, N[e], take * kv[buf][t][e]);
+        nq = fmaf(N[e], qv[buf][t][e], nq);
       }
       nq = wave_sum(nq);
       const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
       if (lane == 0) coef[size_t(t0 + t) * heads + head] = float4{keep, take, 1.0f / den, m};
     }
+  };
+  // (a row's own (li, lf) in coef is read before its place is overwritten: the tile that is walked was requested
+  // a whole tile earlier, and the one requested meanwhile lies behind it)
+  request(r0, 0);
+  for (int t0 = r0; t0 < r1; t0 += 2 * kGateTile) {
+    if (t0 + kGateTile < r1) request(t0 + kGateTile, 1);
+    walk(t0, 0);
+    if (t0 + kGateTile >= r1) break;
+    if (t0 + 2 * kGateTile < r1) request(t0 + 2 * kGateTile, 0);
+    walk(t0 + kGateTile, 1);
   }
 #pragma unroll
-  for (int e = 0; e < kGateMaxPerLane; ++e) {
+  for (int e = 0; e < PER; ++e) {
     const int i = lane + e * kWave;
     if (i < dk) nst[i] = N[e];
   }
@@ -237,8 +251,14 @@ int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const floa
     const long long n = static_cast<long long>(T) * heads;
     mlstm_gate_logs_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, s>>>(ig, ldi, fg, ldf, i_bias, f_bias, cap, cf, n, heads);
   }
-  mlstm_gates_kernel<<<dim3(heads, S), kWave, 0, s>>>(q, ldq, k, ldk, ig, ldi, fg, ldf, i_bias, f_bias, cap, q_scale, cf, n_state,
-                                                      m_state, run_start, seq_start, state_slots, heads, dk, logs_first);
+#define KVCM_MLSTM_GATES(PER)                                                                                                 \
+  mlstm_gates_kernel<PER><<<dim3(heads, S), kWave, 0, s>>>(q, ldq, k, ldk, ig, ldi, fg, ldf, i_bias, f_bias, cap, q_scale, cf, \
+                                                           n_state, m_state, run_start, seq_start, state_slots, heads, dk,    \
+                                                           logs_first)
+  if (dk <= kWave) KVCM_MLSTM_GATES(1);
+  else if (dk <= 2 * kWave) KVCM_MLSTM_GATES(2);
+  else KVCM_MLSTM_GATES(4);
+#undef KVCM_MLSTM_GATES
 #define KVCM_MLSTM(DKP, G, TILE)                                                                                             \
   {                                                                                                                          \
     const int col_blocks = (dv + 256 / G - 1) / (256 / G);                                                                   \

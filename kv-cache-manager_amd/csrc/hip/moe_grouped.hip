@@ -81,15 +81,15 @@ __global__ void __launch_bounds__(256)
     const int r = tid / 8 + 32 * q;
     aok[q] = r < rows;
     const long long src = UP ? pair_of[r] / top : p0 + (aok[q] ? r : 0);
-    arow[q] = A + src * lda + kk;
+    arow[q] = A + src * lda;
     const int c = n0 + r;
     bok[q] = c < N;
-    brow[q] = W + (static_cast<long long>(e) * N + (bok[q] ? c : N - 1)) * K + kk;
+    brow[q] = W + (static_cast<long long>(e) * N + (bok[q] ? c : N - 1)) * K;
   }
   uint4 areg[4], breg[4];
   auto request = [&](int k0) {      // unconditional loads from clamped places, masked afterwards
     const bool kin = k0 + kk < K;      // K is a multiple of 8: a piece lies inside or outside
-    const int off = kin ? k0 : 0;
+    const int off = kin ? k0 + kk : 0;      // (a piece outside is read from the row's start: nothing beyond a row is touched)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const uint4 a = *reinterpret_cast<const uint4*>(arow[q] + off);

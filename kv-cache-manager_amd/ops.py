@@ -3,7 +3,9 @@ the host that their shapes and dtypes are what the kernel assumes, and launches 
 current stream.  There is no fallback: without the library (or without a GPU) these raise.
 """
 import ctypes as C
+import os
 import struct as _struct
+import sys
 import threading
 
 import torch
@@ -242,11 +244,22 @@ def _slots(fn, args):
     return out
 
 
+# KVCM_SYNC_LAUNCHES=1: every launching entry is named on stderr before it is called and waited for after it, so that a
+# kernel's failure is reported at its own call (for hunting faults; steps run many times slower).
+_SYNC_LAUNCHES = bool(int(os.environ.get("KVCM_SYNC_LAUNCHES", "0") or 0))
+
+
 def _call(name, *args):
     """Calls a launching entry; while a program records, notes the call there first."""
     fn = getattr(lib(), name)
     if _recording is not None:
         _recording.add(name, _slots(fn, args))
+    if _SYNC_LAUNCHES:
+        print("[kvcm launch] %s %s" % (name, " ".join(str(a) for a in args if isinstance(a, (int, float)) and abs(a) < 1 << 20)),
+              file=sys.stderr, flush=True)
+        _check(fn(*args))
+        torch.cuda.synchronize()
+        return
     _check(fn(*args))
 
 
