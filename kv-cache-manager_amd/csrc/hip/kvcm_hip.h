@@ -212,7 +212,7 @@ int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const floa
 // (mlstm.hip) a matrix memory with exponential gates, walked token by token
 int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* ig, int ldi,
                     const float* fg, int ldf, const float* i_bias, const float* f_bias, float cap, float q_scale, float* coef,
-                    float* o, int ldo, float* s_state, float* n_state, float* m_state, const int* run_start,
+                    float* n_new, float* o, int ldo, float* s_state, float* n_state, float* m_state, const int* run_start,
                     const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, int T, int max_run,
                     hipStream_t s);
 // (moe.hip) a routed feed-forward: the choice of experts, and the experts' two products a row at a time

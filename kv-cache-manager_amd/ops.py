@@ -103,7 +103,7 @@ def _declare(lib):
     fn("kvcm_scale_rows", vp, C.c_longlong, f, vp)
     fn("kvcm_head_gate", vp, i, i, vp, i, i, i, i, vp)
     fn("kvcm_rms_groups", vp, i, i, i, i, vp, f, i, vp)
-    fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_moe_route", vp, i, i, i, vp, vp, i, vp)
     fn("kvcm_moe_up", vp, i, i, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_moe_down", vp, i, vp, vp, vp, vp, i, i, i, i, i, vp)
@@ -1362,10 +1362,10 @@ def rms_groups(x, col0, size, groups, weight, eps, rows=None):
     return x
 
 
-def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, coef, o, s_state, n_state, m_state, step, heads, dk, dv):
+def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, coef, n_new, o, s_state, n_state, m_state, step, heads, dk, dv):
     """The matrix memory with exponential gates over the step's runs (csrc/hip/mlstm.hip).  q, k [T, heads*dk], v [T, heads*dv],
     gate_in, gate_keep [T, heads] (projections without biases): 32-bit rows; coef: float32 scratch of 4 T heads values;
-    states [slots, heads, dk, dv], [slots, heads, dk], [slots, heads]."""
+    n_new: float32 scratch of seqs heads dk values; states [slots, heads, dk, dv], [slots, heads, dk], [slots, heads]."""
     T = o.shape[0]
     for t, n, c in ((q, "q", heads * dk), (k, "k", heads * dk), (v, "v", heads * dv), (o, "o", heads * dv), (gate_in, "gate_in", heads),
                     (gate_keep, "gate_keep", heads)):
@@ -1374,10 +1374,11 @@ def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, co
     _f32(in_bias, "in_bias", heads)
     _f32(keep_bias, "keep_bias", heads)
     _f32(coef, "coef", 4 * T * heads)
+    _f32(n_new, "n_new", step.seqs * heads * dk)
     for t, n, shape in ((s_state, "s_state", (heads, dk, dv)), (n_state, "n_state", (heads, dk)), (m_state, "m_state", (heads,))):
         _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and tuple(t.shape[1:]) == shape, f"{n} must be float32 [slots, {shape}]")
     _call("kvcm_mlstm_scan", _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(gate_in), gate_in.stride(0),
-          _ptr(gate_keep), gate_keep.stride(0), _ptr(in_bias), _ptr(keep_bias), float(cap), float(q_scale), _ptr(coef), _ptr(o),
+          _ptr(gate_keep), gate_keep.stride(0), _ptr(in_bias), _ptr(keep_bias), float(cap), float(q_scale), _ptr(coef), _ptr(n_new), _ptr(o),
           o.stride(0), _ptr(s_state), _ptr(n_state), _ptr(m_state), _ptr(step.run_start), _ptr(step.seq_start),
           _ptr(step.state_slots), step.seqs, heads, dk, dv, T, int(step.max_run), _stream())
     return o

@@ -179,8 +179,10 @@ class MatrixMemoryMixer(_StatefulMixer):
         at = [0, heads * d, 2 * heads * d, 2 * heads * d + heads * dv, 2 * heads * (d + dv), 2 * heads * (d + dv) + heads]
         q, k, v, g, gi, gf = (proj[:, lo:] for lo in at)
         coef = step.ws("memory_factors", (T, 4 * heads), torch.float32)
+        seqs = max(step.seqs, step.limits.max_seqs if step.limits is not None else step.seqs)
+        n_new = step.flat("memory_normalizer", seqs * heads * d)
         o = step.ws("memory_o", (T, heads * dv), torch.float32)
-        ops.mlstm_scan(q, k, v, gi, gf, w["in_bias"], w["keep_bias"], p["gate_cap"], float(d) ** -0.5, coef, o,
+        ops.mlstm_scan(q, k, v, gi, gf, w["in_bias"], w["keep_bias"], p["gate_cap"], float(d) ** -0.5, coef, n_new, o,
                        self.state("memory"), self.state("normalizer"), self.state("maximum"), step, heads, d, dv)
         gated = step.ws("memory_gated", (T, heads * dv))
         ops.head_norm_gate(o, g, w["norm"], gated, heads, dv, p["eps"])

@@ -247,7 +247,7 @@ def test_matrix_memory_against_the_plain_recurrence(shape):
         q, k, v, gi, gf = (packed[:, lo:] for lo in at)
         coef = torch.empty(st.rows, 4 * heads, device=DEV)
         o = torch.empty(st.rows, heads * dv, device=DEV)
-        ops.mlstm_scan(q, k, v, gi, gf, dev(bi), dev(bf), cap, d ** -0.5, coef, o, S, N, M, st, heads, d, dv)
+        ops.mlstm_scan(q, k, v, gi, gf, dev(bi), dev(bf), cap, d ** -0.5, coef, torch.empty(st.seqs * heads * d, device=DEV), o, S, N, M, st, heads, d, dv)
         r = 0
         for s, p0, c in runs:
             got[s][p0:p0 + c] = o[r:r + c].cpu().numpy()
@@ -278,7 +278,7 @@ def test_matrix_memory_keeps_what_an_open_gate_wrote_long_ago():
         packed = dev(np.concatenate([x[p:p + c].reshape(c, -1) for x in (q, k, v, gi, gf)], 1))
         at = np.cumsum([0, d, d, dv, 1])
         ops.mlstm_scan(*(packed[:, lo:] for lo in at), dev(np.zeros(1)), dev(np.zeros(1)), 40.0, 1.0, torch.empty(c, 4, device=DEV),
-                       o[p:p + c], S, N, M, st, heads, d, dv)
+                       torch.empty(heads * d, device=DEV), o[p:p + c], S, N, M, st, heads, d, dv)
         p += c
     np.testing.assert_allclose(o[-1].cpu().numpy(), v[5, 0], atol=2e-3)
 
