@@ -89,6 +89,8 @@ __device__ __forceinline__ void wave_dots(const float* xs, const T* w, size_t st
     wc[c] = w + size_t(c < cols ? c : cols - 1) * stride;
   }
   if (vec) {
+    // (two trips' pieces on their way at once; four were measured and gained nothing: the walk is bound by its chain of
+    // dependent sums, not by bytes in flight)
 #pragma unroll 2
     for (int k = lane * N; k < K; k += kWave * N) {
       float f[CW][N];

@@ -60,14 +60,19 @@ template <bool UP>
 __global__ void __launch_bounds__(256)
     moe_grouped_kernel(const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, const int* __restrict__ order,
                        const int* __restrict__ tiles, int top, void* __restrict__ out, const float* __restrict__ weight, int N,
-                       int K) {
+                       int K, int col_blocks) {
   __shared__ __attribute__((aligned(16))) uint16_t As[kGM][kGPitch];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[kGN][kGPitch];
   __shared__ int pair_of[kGM];
-  const int tile = blockIdx.x;
-  if (tile >= tiles[0]) return;
+  // The chip hands consecutive workgroups to its eight XCDs in turn, each with an L2 of its own.  Workgroup L goes to
+  // XCD L % 8; it takes a column block that is congruent to its XCD and walks the tiles in order, so that the tiles of
+  // one expert (neighbours in the list) meet the same blocks of that expert's matrix in the same L2.
+  const int col_slots = (col_blocks + 7) / 8;
+  const int xcd = blockIdx.x % 8, turn = blockIdx.x / 8;
+  const int tile = turn / col_slots, col_block = (turn % col_slots) * 8 + xcd;
+  if (col_block >= col_blocks || tile >= tiles[0]) return;
   const int e = tiles[1 + 3 * tile], p0 = tiles[2 + 3 * tile], rows = tiles[3 + 3 * tile];
-  const int n0 = blockIdx.y * kGN;
+  const int n0 = col_block * kGN;
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
   if (tid < kGM) pair_of[tid] = order[p0 + (tid < rows ? tid : 0)];
   __syncthreads();
@@ -188,12 +193,15 @@ int kvcm_moe_grouped(const void* h, int ldh, const void* w_up, const void* w_dow
                    reinterpret_cast<uintptr_t>(w_down) % 16 == 0 && reinterpret_cast<uintptr_t>(act) % 16 == 0,
                "moe_grouped: operands must be 16-byte aligned");
   const int n = T * top, max_tiles = kvcm_moe_grouped_max_tiles(n, E);
-  KVCM_REQUIRE((F + kGN - 1) / kGN <= 65535 && (H + kGN - 1) / kGN <= 65535, "moe_grouped: too many columns");
+  const int up_blocks = (F + kGN - 1) / kGN, down_blocks = (H + kGN - 1) / kGN;
+  const long long up_grid = static_cast<long long>(max_tiles) * ((up_blocks + 7) / 8) * 8;
+  const long long down_grid = static_cast<long long>(max_tiles) * ((down_blocks + 7) / 8) * 8;
+  KVCM_REQUIRE(up_grid < (1ll << 31) && down_grid < (1ll << 31), "moe_grouped: too many tiles");
   moe_group_kernel<<<1, 1024, 2 * E * sizeof(int), s>>>(chosen, n, E, order, tiles, max_tiles);
-  moe_grouped_kernel<true><<<dim3(max_tiles, (F + kGN - 1) / kGN), 256, 0, s>>>(
-      static_cast<const uint16_t*>(h), ldh, static_cast<const uint16_t*>(w_up), order, tiles, top, act, nullptr, F, K);
-  moe_grouped_kernel<false><<<dim3(max_tiles, (H + kGN - 1) / kGN), 256, 0, s>>>(
-      static_cast<const uint16_t*>(act), F, static_cast<const uint16_t*>(w_down), order, tiles, top, y, weight, H, F);
+  moe_grouped_kernel<true><<<static_cast<unsigned>(up_grid), 256, 0, s>>>(
+      static_cast<const uint16_t*>(h), ldh, static_cast<const uint16_t*>(w_up), order, tiles, top, act, nullptr, F, K, up_blocks);
+  moe_grouped_kernel<false><<<static_cast<unsigned>(down_grid), 256, 0, s>>>(
+      static_cast<const uint16_t*>(act), F, static_cast<const uint16_t*>(w_down), order, tiles, top, y, weight, H, F, down_blocks);
   const long long total = static_cast<long long>(T) * H;
   const long long blocks = (total + 255) / 256;
   moe_combine_kernel<<<static_cast<unsigned>(blocks > 16384 ? 16384 : blocks), 256, 0, s>>>(y, out, total, H, top);
