@@ -2,7 +2,7 @@
 
   architecture    "Furapel"
   vocab, width    sizes of the vocabulary and of the residual stream
-  embedding.scale factor on the embedding
+  embedding.scale factor on the embedding (default 1)
   norm.eps        epsilon of the root-mean-square divisions inside mixers (the layers' own norms use none)
   logit_scale     factor on the logits (default 1)
   layers[i]       type: "attention" | "latent_attention" | "mlstm"; mixer: that mixer's sizes;
@@ -11,7 +11,8 @@
                   caches of its own and led in by a product that mixes the stream with the embedding again
 
 Mixers.  attention: heads, kv_heads, dim, vdim, scale, rot {dims, base, scaling {factor, original, fast, slow} or
-absent} (rot absent or dims 0: no rotation).  latent_attention: heads, dim, vdim, kv_rank, scale, mask {size}.
+absent} (rot absent or dims 0: no rotation; kv_heads defaults to heads, vdim to dim, rot.base to 10000).
+latent_attention: heads, dim, vdim, kv_rank, scale, mask {size} (mask absent: every earlier token).
 mlstm: heads, dim, vdim, gate_cap.
 """
 from dataclasses import dataclass
@@ -65,8 +66,10 @@ class LatentAttentionConfig:
     window: int
 
     def to_dict(self):
-        return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "kv_rank": self.kv_rank, "scale": self.scale,
-                "mask": {"size": self.window}}
+        d = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "kv_rank": self.kv_rank, "scale": self.scale}
+        if self.window:
+            d["mask"] = {"size": self.window}
+        return d
 
 
 @dataclass(frozen=True)
@@ -119,7 +122,7 @@ def _attention(problems, w, m):
             rot = {}
         dims = _pos_int(problems, w + ".rot", rot, "dims", allow_zero=True)
         if dims:
-            base = _number(problems, w + ".rot", rot, "base")
+            base = _number(problems, w + ".rot", rot, "base") if "base" in rot else 10000.0
             sc = rot.get("scaling")
             if sc is not None:
                 if not isinstance(sc, dict):
@@ -130,8 +133,9 @@ def _attention(problems, w, m):
                                         _number(problems, ws, sc, "fast"), _number(problems, ws, sc, "slow"))
                 if base == 1.0:
                     problems.append(f"{w}.rot.base 1 cannot be rescaled")
-    cfg = GatedAttentionConfig(heads=_pos_int(problems, w, m, "heads"), kv_heads=_pos_int(problems, w, m, "kv_heads"),
-                               dim=_pos_int(problems, w, m, "dim"), vdim=_pos_int(problems, w, m, "vdim"),
+    heads, dim = _pos_int(problems, w, m, "heads"), _pos_int(problems, w, m, "dim")
+    cfg = GatedAttentionConfig(heads=heads, kv_heads=_pos_int(problems, w, m, "kv_heads") if "kv_heads" in m else heads,
+                               dim=dim, vdim=_pos_int(problems, w, m, "vdim") if "vdim" in m else dim,
                                scale=_number(problems, w, m, "scale"), rot_dims=dims, rot_base=base, scaling=scaling)
     if cfg.heads % cfg.kv_heads:
         problems.append(f"{w}: heads {cfg.heads} is not a multiple of kv_heads {cfg.kv_heads}")
@@ -141,10 +145,15 @@ def _attention(problems, w, m):
 
 
 def _latent(problems, w, m):
-    mask = m.get("mask") if isinstance(m.get("mask"), dict) else {}
-    return LatentAttentionConfig(heads=_pos_int(problems, w, m, "heads"), dim=_pos_int(problems, w, m, "dim"),
-                                 vdim=_pos_int(problems, w, m, "vdim"), kv_rank=_pos_int(problems, w, m, "kv_rank"),
-                                 scale=_number(problems, w, m, "scale"), window=_pos_int(problems, w + ".mask", mask, "size"))
+    mask = m.get("mask")
+    if mask is not None and not isinstance(mask, dict):
+        problems.append(f"{w}.mask must be an object or absent")
+        mask = None
+    dim = _pos_int(problems, w, m, "dim")
+    return LatentAttentionConfig(heads=_pos_int(problems, w, m, "heads"), dim=dim,
+                                 vdim=_pos_int(problems, w, m, "vdim") if "vdim" in m else dim, kv_rank=_pos_int(problems, w, m, "kv_rank"),
+                                 scale=_number(problems, w, m, "scale"),
+                                 window=_pos_int(problems, w + ".mask", mask, "size") if mask is not None else 0)      # no mask: every earlier token
 
 
 def _memory(problems, w, m):
@@ -166,7 +175,7 @@ class FurapelConfig:
     def from_dict(cls, raw: dict) -> "FurapelConfig":
         problems = []
         vocab, width = _pos_int(problems, "config", raw, "vocab"), _pos_int(problems, "config", raw, "width")
-        scale = _number(problems, "embedding", raw.get("embedding"), "scale")
+        scale = _number(problems, "embedding", raw.get("embedding"), "scale") if isinstance(raw.get("embedding"), dict) and "scale" in raw["embedding"] else 1.0
         eps = _number(problems, "norm", raw.get("norm"), "eps")
         logit_scale = _number(problems, "config", raw, "logit_scale", positive=False) if "logit_scale" in raw else 1.0
         layers = []

@@ -35,6 +35,15 @@ def test_configurations_round_trip_and_name_every_bad_key():
     for piece in ("config.width", "kv_heads 3", "rot.dims 7", "layers[1].mixer.mask.size", "'lstm' is not supported", "top 9 exceeds",
                   "loop.times", "are not a stretch"):
         assert piece in text, (piece, text)
+    # what a file may leave out: the embedding's factor, the logit scale, kv_heads (= heads), vdim (= dim), the rotation's
+    # base, the latent attention's mask (then every earlier token is seen)
+    lean = copy.deepcopy(cases.CONFIGS["U"])
+    del lean["embedding"], lean["logit_scale"], lean["layers"][1]["mixer"]["kv_heads"], lean["layers"][1]["mixer"]["vdim"]
+    del lean["layers"][1]["mixer"]["rot"]["base"], lean["layers"][2]["mixer"]["mask"], lean["layers"][2]["mixer"]["vdim"]
+    cfg = FurapelConfig.from_dict(lean)
+    a, l = cfg.layers[1].mixer, cfg.layers[2].mixer
+    assert (cfg.embedding_scale, cfg.logit_scale, a.kv_heads, a.vdim, a.rot_base, l.window, l.vdim) == (1.0, 1.0, 4, 16, 10000.0, 0, 12)
+    assert FurapelConfig.from_dict(cfg.to_dict()) == cfg
     dense = copy.deepcopy(cases.CONFIGS["U"])
     dense["layers"][1]["mlp"]["kind"] = "dense"
     with pytest.raises(ConfigError, match="mlp.kind 'dense' is not supported"):

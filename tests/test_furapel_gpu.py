@@ -130,12 +130,12 @@ def test_stream_packed_with_the_embedding_scaled_logits_head_gates_and_small_nor
     np.testing.assert_allclose(r.cpu().numpy(), want, atol=3e-6)
 
 
-@pytest.mark.parametrize("scaling", [None, (2.0, 2048, 32.0, 1.0), (8.0, 50, 4.0, 0.5), (3.0, 100000, 1000.0, 200.0)])
+@pytest.mark.parametrize("scaling", [None, (2.5, 1024, 24.0, 1.5), (8.0, 50, 4.0, 0.5), (3.0, 100000, 1000.0, 200.0)])
 def test_rescaled_frequencies_and_the_half_split_rotation(scaling):
     from kvcm_amd import ops
     from kvcm_amd.parts.gated_attention_parts import rescaled_frequencies
     rng = np.random.default_rng(2)
-    for dims, d, base in ((8, 16, 100.0), (32, 32, 20000.0), (2, 10, 7.0), (64, 64, 500000.0)):
+    for dims, d, base in ((8, 16, 100.0), (32, 32, 30000.0), (2, 10, 7.0), (64, 64, 500000.0)):
         sc = dict(zip(("factor", "original", "fast", "slow"), scaling)) if scaling else None
         want_f, want_factor = plain.yarn_frequencies(dims, base, sc)
         f, factor = rescaled_frequencies(dims, base, scaling)
