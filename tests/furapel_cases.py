@@ -58,7 +58,7 @@ CONFIGS = {
     "X": {"architecture": "Furapel", "vocab": 200, "width": 96, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
           "loop": {"start": 1, "stop": 2, "times": 1},
           "layers": [_layer(_latent(4, 24, 24, 40, 0.2, 70), 8, 2, 48),
-                     _layer(_attention(6, 2, 128, 128, 0.09, rot=32, base=20000.0, scaling=(4.0, 64, 16.0, 2.0)), 8, 3, 32)]},
+                     _layer(_attention(6, 2, 128, 128, 0.09, rot=32, base=25000.0, scaling=(4.0, 64, 16.0, 2.0)), 8, 3, 32)]},
 }
 BLOCK_SIZE = {"U": 16, "V": 16, "W": 8, "X": 32}
 
