@@ -201,7 +201,8 @@ int kvcm_delta_scan(const float* r, int ldr, const float* k, int ldk, const floa
 
 // (stream_norms.hip) a norm without statistics beside the residual additions of a layer whose mixer and feed-forward run
 // side by side; the stream packed with the embedding for a product; a factor on logits; a gate per head; small norms in place
-int kvcm_dyt_norm(float* x, int use_x, const float* a, const float* b, const int* rows, int write_back, const float* w1,
+int kvcm_dyt_norm(float* x, int use_x, const float* a, int a_splits, long long a_stride, const float* b, const int* rows, int write_back,
+                  const float* w1,
                   const float* b1, float alpha1, void* out1, const float* w2, const float* b2, float alpha2, void* out2,
                   int out_dtype, int R, int H, hipStream_t s);
 int kvcm_stream_pack(const float* x, const float* a, const float* b, const float* x0, void* out, int out_dtype, int T, int H,

@@ -19,15 +19,16 @@ namespace kvcm {
 
 template <class TO>
 __global__ void __launch_bounds__(256)
-    dyt_norm_kernel(float* __restrict__ x, int use_x, const float* __restrict__ a, const float* __restrict__ b,
-                    const int* __restrict__ rows, int write_back, const float* __restrict__ w1,
+    dyt_norm_kernel(float* __restrict__ x, int use_x, const float* __restrict__ a, int a_splits, long long a_stride,
+                    const float* __restrict__ b, const int* __restrict__ rows, int write_back, const float* __restrict__ w1,
                     const float* __restrict__ b1, float alpha1, TO* __restrict__ out1, const float* __restrict__ w2,
                     const float* __restrict__ b2, float alpha2, TO* __restrict__ out2, long long n, int H) {
   for (long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x; idx < n; idx += static_cast<long long>(gridDim.x) * 256) {
     const int r = static_cast<int>(idx / H), c = static_cast<int>(idx % H);
     const size_t src = size_t(rows ? rows[r] : r) * H + c;
     float v = use_x ? x[src] : 0.f;
-    if (a) v += a[src];
+    if (a)
+      for (int sp = 0; sp < a_splits; ++sp) v += a[sp * a_stride + src];      // (the slices of a split product, in split order)
     if (b) v += b[src];
     if (write_back) x[idx] = v;
     if (out1) store_f(out1 + idx, fmaf(tanhf(alpha1 * v), w1[c], b1[c]));
@@ -94,24 +95,26 @@ using namespace kvcm;
 
 extern "C" {
 
-// x [T, H] 32-bit; a, b [T, H] 32-bit or null; rows: source rows of the R outputs (null: row r, and then x <- x + a + b
-// is written back when write_back is set); use_x 0: the sum starts from zero (x is only written).  out1 / out2 [R, H]
-// in out_dtype, each with its weight, bias and factor, or null.
-int kvcm_dyt_norm(float* x, int use_x, const float* a, const float* b, const int* rows, int write_back, const float* w1,
+// x [T, H] 32-bit; a, b [T, H] 32-bit or null; a may be the un-added slices of a split product, [a_splits][T][H] with
+// a_stride floats between slices (a_splits 1: finished); rows: source rows of the R outputs (null: row r, and then
+// x <- x + a + b is written back when write_back is set); use_x 0: the sum starts from zero (x is only written).
+// out1 / out2 [R, H] in out_dtype, each with its weight, bias and factor, or null.
+int kvcm_dyt_norm(float* x, int use_x, const float* a, int a_splits, long long a_stride, const float* b, const int* rows, int write_back, const float* w1,
                   const float* b1, float alpha1, void* out1, const float* w2, const float* b2, float alpha2, void* out2,
                   int out_dtype, int R, int H, hipStream_t s) {
   if (R == 0) return 0;
   KVCM_REQUIRE(R > 0 && H > 0 && x != nullptr, "dyt_norm: bad sizes R=%d H=%d", R, H);
   KVCM_REQUIRE(!(rows && write_back), "dyt_norm: gathered rows are not written back");
   KVCM_REQUIRE(use_x || a, "dyt_norm: nothing to norm");
+  KVCM_REQUIRE(a_splits >= 1 && a_stride >= 0, "dyt_norm: an addition has at least one slice");
   KVCM_REQUIRE((!out1 || (w1 && b1)) && (!out2 || (w2 && b2)), "dyt_norm: an output needs its weight and bias");
   KVCM_REQUIRE(out1 || out2 || write_back, "dyt_norm: nothing to do");
   const long long n = static_cast<long long>(R) * H;
   if (out_dtype == kF32)
-    dyt_norm_kernel<float><<<grid_for(n), 256, 0, s>>>(x, use_x, a, b, rows, write_back, w1, b1, alpha1, static_cast<float*>(out1),
+    dyt_norm_kernel<float><<<grid_for(n), 256, 0, s>>>(x, use_x, a, a_splits, a_stride, b, rows, write_back, w1, b1, alpha1, static_cast<float*>(out1),
                                                        w2, b2, alpha2, static_cast<float*>(out2), n, H);
   else if (out_dtype == kBF16)
-    dyt_norm_kernel<bf16_t><<<grid_for(n), 256, 0, s>>>(x, use_x, a, b, rows, write_back, w1, b1, alpha1, static_cast<bf16_t*>(out1),
+    dyt_norm_kernel<bf16_t><<<grid_for(n), 256, 0, s>>>(x, use_x, a, a_splits, a_stride, b, rows, write_back, w1, b1, alpha1, static_cast<bf16_t*>(out1),
                                                         w2, b2, alpha2, static_cast<bf16_t*>(out2), n, H);
   else KVCM_REQUIRE(false, "dyt_norm: unknown output dtype %d", out_dtype);
   return launch_status("dyt_norm");

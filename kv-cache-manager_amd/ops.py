@@ -98,7 +98,7 @@ def _declare(lib):
     fn("kvcm_rotary_pairs_table", vp, vp, i, i, f, vp)
     fn("kvcm_rotate_store", vp, i, vp, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_rotary_freq_table", vp, vp, vp, i, i, f, vp)
-    fn("kvcm_dyt_norm", vp, i, vp, vp, vp, i, vp, vp, f, vp, vp, vp, f, vp, i, i, i, vp)
+    fn("kvcm_dyt_norm", vp, i, vp, i, C.c_longlong, vp, vp, i, vp, vp, f, vp, vp, vp, f, vp, i, i, i, vp)
     fn("kvcm_stream_pack", vp, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_scale_rows", vp, C.c_longlong, f, vp)
     fn("kvcm_head_gate", vp, i, i, vp, i, i, i, i, vp)
@@ -1293,10 +1293,17 @@ class DytNorm:
 def dyt_norm(x, first=None, out1=None, second=None, out2=None, add_a=None, add_b=None, rows=None, replace=False):
     """x += add_a + add_b (``replace``: x = add_a + add_b), written back unless ``rows`` gathers; then
     out1 = first(x), out2 = second(x), each tanh(alpha x) * weight + bias rounded once to the output's dtype.
-    x, add_a, add_b: float32 [T, H]; out1, out2 [R, H]; rows: int32 [R] source rows (None: row r)."""
+    x, add_a, add_b: float32 [T, H]; out1, out2 [R, H]; rows: int32 [R] source rows (None: row r).  add_a may be the un-added
+    slices of a split product (PartialSums [splits][T][H]): they are added here, in split order."""
     _need(x.dtype == torch.float32 and x.is_contiguous() and x.is_cuda and x.dim() == 2, "x must be contiguous float32 [T, H]")
     T, H = x.shape
-    for t, n in ((add_a, "add_a"), (add_b, "add_b")):
+    a_splits = 1
+    if isinstance(add_a, PartialSums):
+        _need(add_a.rows == T and add_a.cols == H, "an addition's partial sums must match x")
+        add_a, a_splits = add_a.data, add_a.splits
+        _need(add_a.dtype == torch.float32 and add_a.is_contiguous() and add_a.is_cuda and add_a.numel() >= a_splits * T * H,
+              "partial sums must be contiguous float32 [splits][T][H]")
+    for t, n in (((add_a if a_splits == 1 else None), "add_a"), (add_b, "add_b")):
         if t is not None:
             _need(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and tuple(t.shape) == (T, H), f"{n} must match x")
     _need(add_a is not None or add_b is None, "dyt_norm: a second addition needs a first")
@@ -1317,7 +1324,7 @@ def dyt_norm(x, first=None, out1=None, second=None, out2=None, add_a=None, add_b
         _need(R <= T, "x has fewer rows than the output")
     write_back = 1 if (rows is None and add_a is not None) else 0
     _need(write_back or out1 is not None or out2 is not None, "dyt_norm: nothing to do")
-    _call("kvcm_dyt_norm", _ptr(x), 0 if replace else 1, _ptr(add_a), _ptr(add_b), _ptr(rows), write_back,
+    _call("kvcm_dyt_norm", _ptr(x), 0 if replace else 1, _ptr(add_a), a_splits, T * H, _ptr(add_b), _ptr(rows), write_back,
           _ptr(first.weight) if first else 0, _ptr(first.bias) if first else 0, first.alpha if first else 0.0, _ptr(out1),
           _ptr(second.weight) if second else 0, _ptr(second.bias) if second else 0, second.alpha if second else 0.0, _ptr(out2),
           dt, R, H, _stream())

@@ -151,7 +151,7 @@ class GatedAttention(Mixer):
         attn = step.ws("ga_attn", (T, self.nh * self.dv))
         _attend(self, step, q, attn, kc, vc, g, self.nh, self.nkv, self.d, self.dv, p["scale"], p.get("window", 0))
         ops.head_gate(attn, proj[:, self.gate_at:], self.nh, self.dv, rows=T)
-        return linear32(self.ctx, step, attn, w["w_o"], "ga_out")
+        return linear32(self.ctx, step, attn, w["w_o"], "ga_out", keep_partial=True)      # the stream's next norm adds the slices
 
 
 @MIXERS.register("latent_attention")
@@ -211,4 +211,4 @@ class LatentAttention(Mixer):
         ops.rotate_store(proj, q, nh, 1, r, r, rot=0, slots=slots, kcache=kc, vcache=vc, rows=T)
         attn = step.ws("la_attn", (T, nh * r))
         _attend(self, step, q, attn, kc, vc, g, nh, 1, r, r, p["scale"], p.get("window", 0))
-        return linear32(self.ctx, step, attn, w["w_o"], "la_out")
+        return linear32(self.ctx, step, attn, w["w_o"], "la_out", keep_partial=True)

@@ -186,4 +186,4 @@ class MatrixMemoryMixer(_StatefulMixer):
                        self.state("memory"), self.state("normalizer"), self.state("maximum"), step, heads, d, dv)
         gated = step.ws("memory_gated", (T, heads * dv))
         ops.head_norm_gate(o, g, w["norm"], gated, heads, dv, p["eps"])
-        return linear32(self.ctx, step, gated, w["w_o"], "memory_out")
+        return linear32(self.ctx, step, gated, w["w_o"], "memory_out", keep_partial=True)      # the stream's next norm adds the slices

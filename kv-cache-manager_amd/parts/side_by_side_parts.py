@@ -4,16 +4,16 @@ adds both outputs in the launch that norms the stream for the next layer, and a 
 layers in by mixing the stream with the embedding's output again.  Every size, constant and tensor name is a
 parameter.
 """
-import torch
 
 from ..registry import BLOCKS, NORMS, STREAM_PARTS
-from .base import Block, Norm, ParamSpec, Part
+from .base import Block, Norm, ParamSpec, Part, as_tensor
 from .chain_norm_parts import f32_params, linear32
 
 
 class StreamAdditions:
     """Up to two 32-bit sublayer outputs [T, H] that are still to be added to the residual stream: what a
-    side-by-side layer hands to whoever reads the stream next (``dynamic_tanh`` adds them in its own launch)."""
+    side-by-side layer hands to whoever reads the stream next (``dynamic_tanh`` adds them in its own launch).  The first
+    may be the un-added slices of a split product (ops.PartialSums)."""
 
     def __init__(self, a=None, b=None):
         self.a, self.b = (a, b) if a is not None else (b, None)
@@ -88,6 +88,7 @@ class StreamReentry(Part):
         if x0 is None:
             raise RuntimeError("stream_reentry needs the embedding's output: the model's description must set keep_embedding")
         a, b = DynamicTanh._additions(add)
+        a = as_tensor(a) if a is not None else None
         packed = step.ws("reentry_in", (step.rows, 2 * x.shape[1]))
         self.ctx.ops.stream_pack(x, x0, packed, a, b)
         return linear32(self.ctx, step, packed, self.w["w"], "reentry_out")
@@ -105,7 +106,7 @@ class SideBySideResidual(Block):
     def forward(self, step, x, pending):
         p = self.parts
         if pending is not None and not isinstance(pending, StreamAdditions):
-            pending = StreamAdditions(pending if torch.is_tensor(pending) else pending.materialize())
+            pending = StreamAdditions(pending)      # a tensor, or the slices of a split product
         replace = False
         if "reentry" in p:
             pending, replace = StreamAdditions(p["reentry"].forward(step, x, pending)), True

@@ -91,6 +91,19 @@ def test_dynamic_tanh_with_additions_gather_and_replacement():
         ops.dyt_norm(xs, n2, out, add_a=dev(a), replace=True)
         np.testing.assert_allclose(xs.cpu().numpy(), a, atol=1e-6)
         np.testing.assert_allclose(out.cpu().numpy(), plain.dynamic_tanh(a, 1.3, w2, b2), atol=3e-6)
+    # an addition that is still the slices of a split product: they are added here
+    T, H = 3, 200
+    x, sa, b = rng.normal(size=(T, H)), rng.normal(size=(5, T, H)), rng.normal(size=(T, H))
+    w1, b1 = 1.0 + 0.2 * rng.normal(size=H), 0.3 * rng.normal(size=H)
+    n1 = ops.DytNorm(dev(w1), dev(b1), 0.6)
+    xs, out = dev(x), torch.empty(T, H, device=DEV)
+    ops.dyt_norm(xs, n1, out, add_a=ops.PartialSums(dev(sa), 5, T, H, torch.empty(T, H, device=DEV)), add_b=dev(b))
+    np.testing.assert_allclose(xs.cpu().numpy(), x + sa.sum(0) + b, atol=3e-6)
+    np.testing.assert_allclose(out.cpu().numpy(), plain.dynamic_tanh(x + sa.sum(0) + b, 0.6, w1, b1), atol=3e-6)
+    rows = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
+    out = torch.empty(2, H, device=DEV)
+    ops.dyt_norm(dev(x), n1, out, add_a=ops.PartialSums(dev(sa), 5, T, H, torch.empty(T, H, device=DEV)), rows=rows)
+    np.testing.assert_allclose(out.cpu().numpy(), plain.dynamic_tanh(x + sa.sum(0), 0.6, w1, b1)[[2, 0]], atol=3e-6)
     # bfloat16 output: one rounding of the 32-bit result
     out = torch.empty(T, H, device=DEV, dtype=torch.bfloat16)
     ops.dyt_norm(dev(x), n1, out)
